@@ -68,6 +68,7 @@ LIBRARIES: Dict[str, dict] = {
     "latent_attention": {"kind": "hip", "sources": ["kernels/latent_attention.hip"], "headers": ["kernels/common.h", "kernels/score_shape.h"]},
     "scored_attention": {"kind": "hip", "sources": ["kernels/scored_attention.hip"], "headers": ["kernels/common.h", "kernels/score_shape.h"]},
     "gated_recurrence": {"kind": "hip", "sources": ["kernels/gated_recurrence.hip"], "headers": ["kernels/common.h", "kernels/score_shape.h"]},
+    "moe": {"kind": "hip", "sources": ["kernels/moe.hip"], "headers": ["kernels/common.h", "kernels/score_shape.h"]},
     "sampling": {"kind": "hip", "sources": ["kernels/sampling.hip"],
                  "headers": ["kernels/common.h", "kernels/score_shape.h", "kernels/noalloc.h"]},
     "peaks": {"kind": "hip", "sources": ["kernels/peaks.hip"], "headers": ["kernels/common.h", "kernels/score_shape.h"]},
@@ -76,12 +77,12 @@ LIBRARIES: Dict[str, dict] = {
     "engine": {
         "kind": "hiphost",
         "sources": ["engine/ops.cc", "engine/ops_sequence.cc", "engine/ops_scored.cc", "engine/parts.cc", "engine/parts_gated.cc",
-                    "engine/mamba2.cc", "engine/latent_attention.cc", "engine/scored_attention.cc", "engine/recurrent_parts.cc", "engine/json.cc", "engine/weights.cc", "engine/arch.cc",
-                    "engine/gpt2.cc", "engine/kugulorn.cc", "engine/rekirax.cc", "engine/engine.cc", "engine/engine_api.cc"],
+                    "engine/mamba2.cc", "engine/latent_attention.cc", "engine/scored_attention.cc", "engine/recurrent_parts.cc", "engine/linear_attention.cc", "engine/json.cc", "engine/weights.cc", "engine/arch.cc",
+                    "engine/gpt2.cc", "engine/kugulorn.cc", "engine/rekirax.cc", "engine/viladra.cc", "engine/engine.cc", "engine/engine_api.cc"],
         "headers": ["kernels/score_shape.h", "engine/ops.h", "engine/parts.h", "engine/kernels.h", "engine/json.h", "engine/weights.h",
                     "engine/arch.h", "engine/engine.h", "runtime/cache_manager.h", "runtime/scheduler.h"],
         "needs": ["elementwise", "gemm_f32", "gemm_bf16", "attention", "attention_decode", "attention_prefill",
-                  "norm_gate", "ssm", "latent_attention", "scored_attention", "gated_recurrence", "sampling", "runtime"],
+                  "norm_gate", "ssm", "latent_attention", "scored_attention", "gated_recurrence", "moe", "sampling", "runtime"],
     },
     # the command line: a program, not a library (mini_llm_amd/_lib/mini-llm; bin/mini-llm starts it)
     "cli": {

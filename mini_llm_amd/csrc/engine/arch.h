@@ -50,6 +50,7 @@ void register_architecture(const Architecture& a, const std::string& model_type 
 void register_gpt2();              // gpt2.cc
 void register_kugulorn();          // kugulorn.cc
 void register_rekirax();           // rekirax.cc
+void register_viladra();           // viladra.cc
 // Loads a shared library whose initialisers register parts and architectures (dlopen; stays loaded).
 // Also called for every path in the environment variable MINI_LLM_PLUGINS (colon-separated), once.
 void load_plugin(const std::string& path);

@@ -12,7 +12,8 @@ extern "C" {
 
 // elementwise.hip
 int mllm_embed(const int* ids, const int* pos, const void* wte, const void* wpe, float* x, int T, int D,
-               int dtype, const int* src, const int* prev, int n_prev, hipStream_t stream);
+               int dtype, const int* src, const int* prev, int n_prev, hipStream_t stream, float scale = 1.f);
+int mllm_depth_mix(float* x, float* kept, size_t stride, int n_old, const float* w, size_t n, hipStream_t stream);
 int mllm_select_tokens(int* ids, const int* src, const int* prev, int n, int n_prev, hipStream_t stream);
 int mllm_reset_state(void* state, size_t slot_bytes, int n_slots, const int* slots, const int* starts, int B,
                      hipStream_t stream);
@@ -69,6 +70,9 @@ int mllm_prefill_attention_bf16(const void* q, int q_stride, int q_col, const vo
 // norm_gate.hip
 int mllm_rmsnorm(const float* x, int ldx, const int* rows, const float* w, const float* gate, int ldg, void* y, int ldy,
                  int n, int D, int groups, float eps, int out_dtype, int parts, size_t part_stride, hipStream_t stream);
+int mllm_rmsnorm_gate_after(const float* x, int ldx, const float* w, const float* gate, int ldg, void* y, int ldy, int n, int D, int groups,
+                            float eps, int out_dtype, int parts, size_t part_stride, hipStream_t stream);
+int mllm_softcap(float* x, size_t n, float cap, hipStream_t stream);
 int mllm_rmsnorm_add(float* y, const float* w, const float* scale, float mult, float eps, float* x, int n, int D,
                      int clear, hipStream_t stream);
 int mllm_rmsnorm_add_many(const float* y, size_t y_stride, const float* w, size_t w_stride, int n_in, float mult, float eps,
@@ -118,7 +122,8 @@ int mllm_qk_prepare(const float* proj, int ld, int q_col, int k_col, int v_col, 
 int mllm_scored_attention_rows(const void* q, int ldq, const void* k_pages, const void* v_pages, const int* block_tables,
                                int max_blocks, const int* token_seq, const int* positions, int n_tokens, int H, int G, int d,
                                int dv, int page_size, float scale, float softcap, int window, int chunk, const float* r1,
-                               const float* r2, const float* gate, int ldg, void* out, int ldo, int dtype, hipStream_t stream);
+                               const float* r2, const float* gate, int ldg, void* out, int ldo, int dtype, hipStream_t stream,
+                               int sigmoid_weights = 0, const float* score_bias = nullptr, int gate_per_head = 0);
 
 int mllm_gate_mul(void* x, int ldx, const float* gate, int ldg, int T, int N, int dtype, hipStream_t stream);
 
@@ -128,10 +133,24 @@ int mllm_hgrn2_scan(const float* proj, int ld, int q_col, int f_col, int v_col, 
                     const int* cu_q, const int* state_slots, float* state, size_t slot_floats, size_t state_offset, float* y, int ldy,
                     size_t part_stride, int T, int B, int max_q_len, int H, int d, int dv, int write, float* workspace,
                     hipStream_t stream);
+int mllm_decay_scan(const float* proj, int ld, int q_col, int k_col, int v_col, const float* decay, int ldd, const float* head_decay,
+                    float q_scale, float k_scale, const int* cu_q, const int* state_slots, float* state, size_t slot_floats,
+                    size_t state_offset, float* y, int ldy, size_t part_stride, int T, int B, int max_q_len, int H, int d, int dv, int write,
+                    float* workspace, hipStream_t stream);
+int mllm_rotary_rows(float* proj, int ld, int col0, int T, int n_heads, int d, int rot_dims, double base, const int* positions,
+                     hipStream_t stream);
+int mllm_lowrank_decay(const float* proj, int ld, int a_col, int rank, const float* w, const float* bias, float tau, float* out, int ldo,
+                       int T, int N, hipStream_t stream);
 size_t mllm_hgrn2_workspace_floats(int T, int B, int H, int d, int dv);
 int mllm_hgrn2_chunk();
 int mllm_concat_cast(const float* a, const float* b, int T, int D, void* out, int dtype, hipStream_t stream);
 int mllm_glu_act(const void* gu, int ld, int T, int F, int act, void* out, int ldo, int dtype, hipStream_t stream);
+
+// moe.hip
+int mllm_moe_route(const void* h, int ldh, int dtype, const float* w, int T, int D, int E, int top, float scale, float* weights, int ldw,
+                   hipStream_t stream);
+int mllm_moe_act(const void* up, int ldu, const float* weights, int ldw, int E, int ff, int shared_ff, void* out, int ldo, int T, int dtype,
+                 hipStream_t stream);
 
 // sampling.hip
 int mllm_argmax_chunks(int V);

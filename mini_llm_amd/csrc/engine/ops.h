@@ -133,8 +133,9 @@ struct FedTokens {
 };
 
 // -- the ops -----------------------------------------------------------------------------------------
+// out[t, :] = scale * wte[ids[t], :] (+ wpe[positions[t], :])
 void embed(const int* ids, const int* positions, const Tensor2& wte, const Tensor2* wpe, const Tensor2& out,
-           hipStream_t stream, const FedTokens* fed = nullptr);
+           hipStream_t stream, const FedTokens* fed = nullptr, float scale = 1.f);
 void select_tokens(int* ids, const int* src, const int* prev, int n, int n_prev, hipStream_t stream);
 void reset_state(void* state, size_t slot_bytes, int n_slots, const int* slots, const int* starts, int n_seqs,
                  hipStream_t stream);
@@ -269,6 +270,11 @@ struct ScoredShape {
     float eps = 1e-6f;
     int rot_dims = 0;                          // the first rot_dims columns of a head are turned (half-split pairs)
     double rot_base = 10000.0;
+    // weights without a softmax: a visible key's weight is sigmoid(score + score_bias[h]) (score_bias per head, or
+    // null), not normalised over the keys
+    bool sigmoid_weights = false;
+    const float* score_bias = nullptr;
+    bool gate_per_head = false;                // the gate has one column per head instead of one per value column
 };
 // From the fp32 rows of the input projection (queries at q_col, keys at k_col, values at v_col; v_col < 0: the
 // values are the keys before their norm): q [T, heads * dim] normed and turned, and the keys and values written
@@ -301,6 +307,38 @@ void hgrn2_scan(const Tensor2& proj, int q_col, int f_col, int v_col, const floa
 int hgrn2_parts(int dim);
 int hgrn2_chunk();
 size_t hgrn2_workspace_floats(int tokens, int n_seqs, int heads, int dim, int value_dim);
+// -- linear attention with a decay ------------------------------------------------------------------
+// Per head S <- diag(f) S + k v^T, o = S^T q with q = q_scale * proj[q_col..], k = k_scale * proj[k_col..] (heads * dim
+// each) and v = proj[v_col..] (heads * value_dim) from proj's fp32 rows. The decays f come per token and channel from
+// `decay` ([T, heads * dim] fp32) or, if that is null, one per head from `head_decay` ([heads] fp32, on the device).
+// Shares of y, state, chunks and workspace as for hgrn2_scan (the same kernels; hgrn2_parts, hgrn2_chunk and
+// hgrn2_workspace_floats give the sizes).
+void decay_scan(const Tensor2& proj, int q_col, int k_col, int v_col, const Tensor2* decay, const float* head_decay, float q_scale,
+                float k_scale, const StateArgs& st, size_t state_offset, int heads, int dim, int value_dim, const Tensor2& y,
+                float* workspace, size_t workspace_floats, hipStream_t stream);
+// The first rot_dims columns of n_heads heads of `dim` columns, from column col0 of proj's fp32 rows, turned in place by
+// the tokens' positions (column i pairs with i + rot_dims / 2, angle p * base^(-2i / rot_dims)).
+void rotary_rows(const Tensor2& proj, int col0, int n_heads, int dim, int rot_dims, double base, const int* positions, hipStream_t stream);
+// out[t, c] = sigmoid(w[c, :] . proj[t, a_col : a_col + rank] + bias[c])^(1 / tau): w [N, rank] fp32, out [T, N] fp32.
+void lowrank_decay(const Tensor2& proj, int a_col, const Tensor2& w, const float* bias, float tau, const Tensor2& out, hipStream_t stream);
+// out = rmsnorm(x) * weight * silu(gate[:, gate_col ..]) in `groups` equal parts of the columns, the gate BEHIND the norm
+// (weight [x.cols] or null; gate fp32 rows). Parts as for rmsnorm.
+void rmsnorm_gate_after(const Tensor2& x, const float* weight, float eps, int groups, const Tensor2& gate, int gate_col, const Tensor2& out,
+                        hipStream_t stream, int parts = 1, size_t part_stride = 0);
+// x <- cap tanh(x / cap) (contiguous fp32)
+void softcap(const Tensor2& x, float cap, hipStream_t stream);
+// `kept` holds n_old earlier streams of x's shape one behind the other ([>= (n_old + 1) * rows, cols] fp32, contiguous).
+// x is stored behind them as stream n_old, and x <- sum_(j <= n_old) w[j] stream_j (w: n_old + 1 floats on the device).
+void depth_mix(const Tensor2& x, const Tensor2& kept, int n_old, const float* w, hipStream_t stream);
+
+// -- mixture of experts -----------------------------------------------------------------------------
+// weights[t, e] = scale * softmax(w h_t)[e] for the `top` experts with the largest scores (the lower index wins a tie),
+// 0 for the others. h [T, D] in its dtype, w [E, D] fp32, weights [T, E] fp32.
+void moe_route(const Tensor2& h, const Tensor2& w, int top, float scale, const Tensor2& weights, hipStream_t stream);
+// out[t, e * ff + j] = weights[t, e] * relu(up[t, e * ff + j])^2 for n_experts experts of ff columns; the columns behind
+// them (a shared expert's) are relu(.)^2 alone. out may be up.
+void moe_act(const Tensor2& up, const Tensor2* weights, int n_experts, int ff, const Tensor2& out, hipStream_t stream);
+
 // out = [a | b] row by row in out's dtype (a, b fp32 [T, D])
 void concat_cast(const Tensor2& a, const Tensor2& b, const Tensor2& out, hipStream_t stream);
 // out[t, j] = act(gu[t, j]) * gu[t, F + j] (act: GELU_TANH)

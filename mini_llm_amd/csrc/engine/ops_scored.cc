@@ -122,14 +122,14 @@ void scored_attention(const Tensor2& q, const Tensor2& k_pages, const Tensor2& v
     int ldg = 0;
     if (gate != nullptr) {
         need_f32(*gate, "scored_attention: the gate");
-        if (gate->rows != q.rows || gate_col < 0 || gate_col + no > gate->cols) fail("scored_attention: the gate's columns lie outside its rows");
+        if (gate->rows != q.rows || gate_col < 0 || gate_col + (sh.gate_per_head ? sh.n_heads : no) > gate->cols) fail("scored_attention: the gate's columns lie outside its rows");
         g = static_cast<const float*>(gate->data) + gate_col;
         ldg = i32(gate->stride);
     }
     // keys and values of one width: the kernels that every attention of the engine runs on (tiles of queries for
     // prompt portions, split keys for single tokens), with the shaping handed on; they fall back by themselves to
     // the one-wavefront-per-row kernel below for sizes they do not take
-    if (tuning().scored_shared_kernels && sh.dim == sh.value_dim && sh.dim % 8 == 0 && sh.dim <= 256 && (q.stride * q.esz()) % 16 == 0 && (sh.dim * q.esz()) % 16 == 0 &&
+    if (tuning().scored_shared_kernels && !sh.sigmoid_weights && !sh.gate_per_head && sh.dim == sh.value_dim && sh.dim % 8 == 0 && sh.dim <= 256 && (q.stride * q.esz()) % 16 == 0 && (sh.dim * q.esz()) % 16 == 0 &&
         (reinterpret_cast<uintptr_t>(q.data) & 15) == 0 && (g == nullptr || (ldg % 4 == 0 && (reinterpret_cast<uintptr_t>(g) & 15) == 0)) &&
         step.cu_q != nullptr && step.ctx_len != nullptr && step.n_seqs > 0) {
         const MllmScoreShape shape{sh.softcap, sh.chunk, sh.r1, sh.r2};
@@ -145,7 +145,8 @@ void scored_attention(const Tensor2& q, const Tensor2& k_pages, const Tensor2& v
     }
     check(mllm_scored_attention_rows(q.data, i32(q.stride), k_pages.data, v_pages.data, step.block_tables, step.max_blocks, step.token_seq,
                                      step.positions, i32(q.rows), sh.n_heads, sh.n_kv_heads, sh.dim, sh.value_dim, step.page_size, sh.scale,
-                                     sh.softcap, sh.window, sh.chunk, sh.r1, sh.r2, g, ldg, out.data, i32(out.stride), q.dtype, stream),
+                                     sh.softcap, sh.window, sh.chunk, sh.r1, sh.r2, g, ldg, out.data, i32(out.stride), q.dtype, stream,
+                                     sh.sigmoid_weights ? 1 : 0, sh.score_bias, sh.gate_per_head ? 1 : 0),
           "scored_attention");
 }
 
@@ -175,6 +176,108 @@ void hgrn2_scan(const Tensor2& proj, int q_col, int f_col, int v_col, const floa
     check(mllm_hgrn2_scan(static_cast<const float*>(proj.data), i32(proj.stride), q_col, f_col, v_col, f_bias, lower, st.cu_q, st.state_slots,
                           st.state, st.slot_floats, state_offset, static_cast<float*>(y.data), i32(y.stride), static_cast<size_t>(y.rows) * y.stride,
                           T, st.n_seqs, max_q, heads, dim, value_dim, st.write ? 1 : 0, workspace, stream), "hgrn2_scan");
+}
+
+void decay_scan(const Tensor2& proj, int q_col, int k_col, int v_col, const Tensor2* decay, const float* head_decay, float q_scale,
+                float k_scale, const StateArgs& st, size_t state_offset, int heads, int dim, int value_dim, const Tensor2& y,
+                float* workspace, size_t workspace_floats, hipStream_t stream) {
+    need_f32(proj, "decay_scan: the projection");
+    need_f32(y, "decay_scan: y");
+    if (heads < 1 || dim < 1 || value_dim < 1) fail("decay_scan: heads and sizes must be positive");
+    const int64_t nq = static_cast<int64_t>(heads) * dim, nv = static_cast<int64_t>(heads) * value_dim;
+    if (q_col < 0 || q_col + nq > proj.cols || k_col < 0 || k_col + nq > proj.cols || v_col < 0 || v_col + nv > proj.cols)
+        fail("decay_scan: queries, keys or values lie outside the projection's rows of %lld", (long long)proj.cols);
+    if (y.rows != proj.rows || y.cols != nv) fail("decay_scan: y must be [%lld, %lld]", (long long)proj.rows, (long long)nv);
+    if (decay != nullptr) {
+        need_f32(*decay, "decay_scan: the decays");
+        if (decay->rows != proj.rows || decay->cols != nq) fail("decay_scan: the decays must be [%lld, %lld]", (long long)proj.rows, (long long)nq);
+    } else if (head_decay == nullptr) {
+        fail("decay_scan: decays per token and channel, or one per head, are needed");
+    }
+    check_state(st, state_offset + static_cast<size_t>(heads) * dim * value_dim, "decay_scan");
+    const int T = i32(proj.rows);
+    const int max_q = st.max_q_len > 0 ? st.max_q_len : T;
+    if (workspace != nullptr && workspace_floats < hgrn2_workspace_floats(T, st.n_seqs, heads, dim, value_dim))
+        fail("decay_scan: the workspace holds %zu floats, %zu are needed", workspace_floats, hgrn2_workspace_floats(T, st.n_seqs, heads, dim, value_dim));
+    check(mllm_decay_scan(static_cast<const float*>(proj.data), i32(proj.stride), q_col, k_col, v_col, decay ? static_cast<const float*>(decay->data) : nullptr,
+                          decay ? i32(decay->stride) : 0, head_decay, q_scale, k_scale, st.cu_q, st.state_slots, st.state, st.slot_floats, state_offset,
+                          static_cast<float*>(y.data), i32(y.stride), static_cast<size_t>(y.rows) * y.stride, T, st.n_seqs, max_q, heads, dim, value_dim,
+                          st.write ? 1 : 0, workspace, stream), "decay_scan");
+}
+
+void rotary_rows(const Tensor2& proj, int col0, int n_heads, int dim, int rot_dims, double base, const int* positions, hipStream_t stream) {
+    need_f32(proj, "rotary_rows: the projection");
+    if (n_heads < 1 || dim < 1 || col0 < 0 || col0 + static_cast<int64_t>(n_heads) * dim > proj.cols) fail("rotary_rows: the heads lie outside the projection's rows");
+    if (rot_dims < 0 || rot_dims % 2 != 0 || rot_dims > dim || (rot_dims > 0 && !(base > 0))) fail("rotary_rows: %d turned columns of %d (even, at most the head) and a positive base are needed", rot_dims, dim);
+    if (positions == nullptr) fail("rotary_rows: positions are needed");
+    check(mllm_rotary_rows(static_cast<float*>(proj.data), i32(proj.stride), col0, i32(proj.rows), n_heads, dim, rot_dims, base, positions, stream), "rotary_rows");
+}
+
+void lowrank_decay(const Tensor2& proj, int a_col, const Tensor2& w, const float* bias, float tau, const Tensor2& out, hipStream_t stream) {
+    need_f32(proj, "lowrank_decay: the projection");
+    need_f32(w, "lowrank_decay: the map");
+    need_f32(out, "lowrank_decay: out");
+    if (!w.contiguous() || w.cols < 1 || a_col < 0 || a_col + w.cols > proj.cols) fail("lowrank_decay: the low-rank values lie outside the projection's rows");
+    if (out.rows != proj.rows || out.cols != w.rows) fail("lowrank_decay: out must be [%lld, %lld]", (long long)proj.rows, (long long)w.rows);
+    if (!(tau > 0.f)) fail("lowrank_decay: tau must be positive");
+    check(mllm_lowrank_decay(static_cast<const float*>(proj.data), i32(proj.stride), a_col, i32(w.cols), static_cast<const float*>(w.data), bias, tau,
+                             static_cast<float*>(out.data), i32(out.stride), i32(proj.rows), i32(w.rows), stream), "lowrank_decay");
+}
+
+void rmsnorm_gate_after(const Tensor2& x, const float* weight, float eps, int groups, const Tensor2& gate, int gate_col, const Tensor2& out,
+                        hipStream_t stream, int parts, size_t part_stride) {
+    need_f32(x, "rmsnorm_gate_after: x");
+    need_f32(gate, "rmsnorm_gate_after: the gate");
+    need_act(out, "rmsnorm_gate_after: out");
+    if (groups < 1 || x.cols % groups != 0) fail("rmsnorm_gate_after: %lld columns in %d groups", (long long)x.cols, groups);
+    if (out.rows != x.rows || out.cols != x.cols || gate.rows != x.rows || gate_col < 0 || gate_col + x.cols > gate.cols)
+        fail("rmsnorm_gate_after: out and the gate's columns must match x [%lld, %lld]", (long long)x.rows, (long long)x.cols);
+    check(mllm_rmsnorm_gate_after(static_cast<const float*>(x.data), i32(x.stride), weight, static_cast<const float*>(gate.data) + gate_col, i32(gate.stride),
+                                  out.data, i32(out.stride), i32(x.rows), i32(x.cols), groups, eps, out.dtype, parts, part_stride, stream), "rmsnorm_gate_after");
+}
+
+void softcap(const Tensor2& x, float cap, hipStream_t stream) {
+    need_f32(x, "softcap: x");
+    if (!x.contiguous()) fail("softcap: x must be contiguous");
+    if (!(cap > 0.f)) fail("softcap: the cap must be positive");
+    check(mllm_softcap(static_cast<float*>(x.data), static_cast<size_t>(x.rows) * x.cols, cap, stream), "softcap");
+}
+
+void depth_mix(const Tensor2& x, const Tensor2& kept, int n_old, const float* w, hipStream_t stream) {
+    need_f32(x, "depth_mix: x");
+    need_f32(kept, "depth_mix: the kept streams");
+    if (!x.contiguous() || !kept.contiguous() || kept.cols != x.cols || n_old < 0 || kept.rows < x.rows * (n_old + 1))
+        fail("depth_mix: %d kept streams and the new one do not fit [%lld, %lld]", n_old, (long long)kept.rows, (long long)kept.cols);
+    if (w == nullptr) fail("depth_mix: the weights are missing");
+    check(mllm_depth_mix(static_cast<float*>(x.data), static_cast<float*>(kept.data), static_cast<size_t>(x.rows) * x.cols, n_old, w,
+                         static_cast<size_t>(x.rows) * x.cols, stream), "depth_mix");
+}
+
+void moe_route(const Tensor2& h, const Tensor2& w, int top, float scale, const Tensor2& weights, hipStream_t stream) {
+    need_act(h, "moe_route: h");
+    need_f32(w, "moe_route: the router");
+    need_f32(weights, "moe_route: the weights");
+    if (!w.contiguous() || w.cols != h.cols || weights.rows != h.rows || weights.cols != w.rows) fail("moe_route: the router must be [E, %lld] and the weights [%lld, E]", (long long)h.cols, (long long)h.rows);
+    if (top < 1 || top > w.rows) fail("moe_route: %d of %lld experts", top, (long long)w.rows);
+    check(mllm_moe_route(h.data, i32(h.stride), h.dtype, static_cast<const float*>(w.data), i32(h.rows), i32(h.cols), i32(w.rows), top, scale,
+                         static_cast<float*>(weights.data), i32(weights.stride), stream), "moe_route");
+}
+
+void moe_act(const Tensor2& up, const Tensor2* weights, int n_experts, int ff, const Tensor2& out, hipStream_t stream) {
+    need_act(up, "moe_act: up");
+    if (out.dtype != up.dtype || out.rows != up.rows || out.cols != up.cols) fail("moe_act: out must have up's shape and dtype");
+    if (n_experts < 0 || ff < 1 || static_cast<int64_t>(n_experts) * ff > up.cols) fail("moe_act: %d experts of %d columns do not fit rows of %lld", n_experts, ff, (long long)up.cols);
+    const float* wp = nullptr;
+    int ldw = 0;
+    if (n_experts > 0) {
+        if (weights == nullptr) fail("moe_act: the experts' weights are missing");
+        need_f32(*weights, "moe_act: the weights");
+        if (weights->rows != up.rows || weights->cols != n_experts) fail("moe_act: the weights must be [%lld, %d]", (long long)up.rows, n_experts);
+        wp = static_cast<const float*>(weights->data);
+        ldw = i32(weights->stride);
+    }
+    check(mllm_moe_act(up.data, i32(up.stride), wp, ldw, n_experts, ff, i32(up.cols) - n_experts * ff, out.data, i32(out.stride), i32(up.rows), up.dtype, stream),
+          "moe_act");
 }
 
 void concat_cast(const Tensor2& a, const Tensor2& b, const Tensor2& out, hipStream_t stream) {

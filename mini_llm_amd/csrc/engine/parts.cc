@@ -408,31 +408,35 @@ private:
 };
 
 // x[t,:] = table[id[t],:] (+ the position table's row), into the fp32 stream.
+// Parameter scale (optional): the row is multiplied by it.
 class TokenTable final : public Embedding {
 public:
-    explicit TokenTable(const Params& p) : table_(p.weights("table")) {}
+    explicit TokenTable(const Params& p) : table_(p.weights("table")), scale_(static_cast<float>(p.number("scale", 1.0))) {}
     int vocab_size() const override { return static_cast<int>(table_.rows); }
     int hidden_size() const override { return static_cast<int>(table_.cols); }
     void forward(const StepView& step, const PositionEncoding* position, const Tensor2& x, hipStream_t s) const override {
-        embed(step.token_ids, step.positions, table_, position ? position->table() : nullptr, x, s, &step.fed);
+        embed(step.token_ids, step.positions, table_, position ? position->table() : nullptr, x, s, &step.fed, scale_);
     }
     bool resolves_fed_tokens() const override { return true; }
 
 private:
     Tensor2 table_;         // [V, D]
+    float scale_ = 1.f;
 };
 
-// logits = norm(x[rows]) W^T (+ b), fp32. `weight` is [V, D]: a tied head is handed the embedding's table
+// logits = norm(x[rows]) W^T (+ b), fp32; with the parameter softcap > 0, logits <- softcap tanh(logits / softcap). `weight` is [V, D]: a tied head is handed the embedding's table
 // and reads it in place as the [N, K] operand (the reference builds a transposed copy:
 // /root/reference/src/model/gpt2_model.cu:87-113); an untied head owns its matrix.
 class LinearHead final : public Head {
 public:
-    explicit LinearHead(const Params& p) : lin_(p.weights("weight"), p.weights_or_null("bias")), dtype_(p.integer("dtype")) {}
+    explicit LinearHead(const Params& p)
+        : lin_(p.weights("weight"), p.weights_or_null("bias")), dtype_(p.integer("dtype")), softcap_(static_cast<float>(p.number("softcap", 0.0))) {}
     int vocab_size() const override { return lin_.out_features(); }
     void forward(const Tensor2& x, const Norm& final_norm, const int* rows, const Tensor2& logits, Arena& arena,
                  hipStream_t s) const override {
         // (the norm gathers the wanted rows and, where the kernels allow, is fused into the product)
         final_norm.linear(x, lin_, logits, STORE_F32, rows, nullptr, arena, s);
+        if (softcap_ > 0.f) softcap(logits, softcap_, s);
     }
     size_t workspace_bytes(int rows) const override {
         return static_cast<size_t>(rows) * lin_.in_features() * dtype_size(dtype_) + 512;
@@ -445,6 +449,7 @@ public:
 private:
     Linear lin_;
     int dtype_ = BF16;
+    float softcap_ = 0.f;
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -492,6 +497,7 @@ void register_builtin_parts() {
     register_latent_attention();
     register_scored_attention();
     register_recurrent_parts();
+    register_linear_attention_parts();
 }
 }  // namespace
 
@@ -557,7 +563,8 @@ std::unique_ptr<Block> build_block(const std::string& kind, std::unique_ptr<Mixe
 static void check_order(const DecoderModel& m) {
     if (!m.embedding || !m.head || !m.final_norm) fail("a model needs an embedding, a final norm and a head");
     for (const LayerCall& c : m.order)
-        if (c.layer < 0 || c.layer >= static_cast<int>(m.layers.size()) || c.cache < 0 || c.before >= static_cast<int>(m.stream_steps.size()))
+        if (c.layer < 0 || c.layer >= static_cast<int>(m.layers.size()) || c.cache < 0 || c.before >= static_cast<int>(m.stream_steps.size()) ||
+            c.after >= static_cast<int>(m.stream_steps.size()))
             fail("the execution order names layer %d / cache %d / stream step %d, the model has %zu layers and %zu stream steps", c.layer,
                  c.cache, c.before, m.layers.size(), m.stream_steps.size());
 }
@@ -613,6 +620,12 @@ StepCost DecoderModel::cost() const {
             if (call.pass == 0) c.weight_bytes += st.weight_bytes;
             c.flops_per_token += st.flops_per_token;
         }
+        if (call.after >= 0) {
+            StepCost st;
+            stream_steps[call.after]->add_cost(st);
+            if (call.after_pass == 0) c.weight_bytes += st.weight_bytes;
+            c.flops_per_token += st.flops_per_token;
+        }
     }
     final_norm->add_cost(c);
     head->add_cost(c);
@@ -630,6 +643,11 @@ size_t DecoderModel::workspace_bytes(int tokens, int n_logits) const {
     for (const auto& st : stream_steps) {
         if (st->wants_embedding_output()) { stream += one; break; }
     }
+    {
+        int kept = 0;
+        for (const auto& st : stream_steps) kept = std::max(kept, st->kept_streams());
+        stream += one * static_cast<size_t>(kept);
+    }
     for (const auto& st : stream_steps) per_layer = std::max(per_layer, st->workspace_bytes(tokens));
     const int rows = std::max(n_logits, 1);
     const size_t at_head = head->workspace_bytes(rows) + 2 * final_norm->workspace_bytes(rows);
@@ -645,10 +663,14 @@ void DecoderModel::forward(const StepView& step, const std::vector<CacheView>& c
     Tensor2 x = arena.tensor(F32, step.n_tokens, hidden_size());
     embedding->forward(step, position.get(), x, s);
     // a stream step that mixes the embedding's output back in later: a copy of it stays for the step
-    Tensor2 x0;
+    // (with room behind it for the streams that a stream step keeps for itself during the step)
+    Tensor2 x0, x0_and_kept;
+    int kept = 0;
+    for (const auto& st : stream_steps) kept = std::max(kept, st->kept_streams());
     for (const auto& st : stream_steps) {
         if (!st->wants_embedding_output()) continue;
-        x0 = arena.tensor(F32, step.n_tokens, hidden_size());
+        x0_and_kept = arena.tensor(F32, static_cast<int64_t>(step.n_tokens) * (1 + kept), hidden_size());
+        x0 = x0_and_kept.row_range(0, step.n_tokens);
         if (hipMemcpyAsync(x0.data, x.data, static_cast<size_t>(step.n_tokens) * hidden_size() * 4, hipMemcpyDeviceToDevice, s) != hipSuccess)
             fail("the copy of the embedding's output failed");
         break;
@@ -668,11 +690,19 @@ void DecoderModel::forward(const StepView& step, const std::vector<CacheView>& c
         times.set_layer(c.layer);
         if (c.before >= 0) {
             const size_t mark = arena.mark();
-            stream_steps[c.before]->forward(x, x0, c.pass, with_rows, arena, s);
+            const StreamStep& st = *stream_steps[c.before];
+            st.forward(x, st.kept_streams() > 0 ? x0_and_kept : x0, c.pass, with_rows, arena, s);
             arena.release(mark);
             times.mark("stream_step", s);
         }
         layers[c.layer]->forward(x, with_rows, caches[c.cache], c.write, arena, s);
+        if (c.after >= 0) {
+            const size_t mark = arena.mark();
+            const StreamStep& st = *stream_steps[c.after];
+            st.forward(x, st.kept_streams() > 0 ? x0_and_kept : x0, c.after_pass, with_rows, arena, s);
+            arena.release(mark);
+            times.mark("stream_step_after", s);
+        }
     }
     times.set_layer(-1);
     if (step.n_logits == 0) { times.end_step(s); return; }

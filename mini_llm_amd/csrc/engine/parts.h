@@ -265,6 +265,12 @@ class FeedForward {
 public:
     virtual ~FeedForward() = default;
     virtual void forward(NormedInput& h, const StepView& step, const Tensor2& x, Arena& arena, hipStream_t s) const = 0;
+    // The same, but x is SET to the result (x need not hold anything before). A feed-forward whose last product can
+    // store instead of add overrides this; otherwise x is cleared first.
+    virtual void forward_set(NormedInput& h, const StepView& step, const Tensor2& x, Arena& arena, hipStream_t s) const {
+        fill_zero(x, s);
+        forward(h, step, x, arena, s);
+    }
     virtual size_t workspace_bytes(int tokens) const = 0;
     virtual void reserve(int max_seqs, hipStream_t s) const { (void)max_seqs; (void)s; }
     virtual void add_cost(StepCost&) const {}
@@ -285,14 +291,17 @@ public:
 };
 
 // Something that happens to the whole stream between two layers (an entry of the execution order names it
-// with `before`): x is the stream, x0 the embedding's output of the same step, `pass` the number the entry gives
-// (a group of layers that runs several times counts its runs).
+// with `before` or `after`): x is the stream, x0 the embedding's output of the same step, `pass` the number the entry
+// gives (a group of layers that runs several times counts its runs). A step that keeps streams of its own for the
+// step (kept_streams() > 0) is handed x0 with that many more blocks of x's rows behind the embedding's output:
+// room that is its own from one call to the next within a step.
 class StreamStep {
 public:
     virtual ~StreamStep() = default;
     virtual void forward(const Tensor2& x, const Tensor2& x0, int pass, const StepView& step, Arena& arena, hipStream_t s) const = 0;
     virtual size_t workspace_bytes(int tokens) const = 0;
     virtual bool wants_embedding_output() const { return false; }
+    virtual int kept_streams() const { return 0; }         // > 0 goes with wants_embedding_output()
     virtual void reserve(int max_seqs, hipStream_t s) const { (void)max_seqs; (void)s; }
     virtual void add_cost(StepCost&) const {}
 };
@@ -351,6 +360,10 @@ void register_latent_attention();
 // (recurrent_parts.cc).
 void register_scored_attention();
 void register_recurrent_parts();
+// Linear attention with a decay, the feed-forward of routed experts, the stream step that hands on a weighted sum of
+// all streams so far (linear_attention.cc); the arrangement with a norm behind each sub-layer only is registered with
+// the gated parts.
+void register_linear_attention_parts();
 
 // One entry of the execution order: which layer runs, on which cache, and whether it writes it.
 struct LayerCall {
@@ -358,6 +371,8 @@ struct LayerCall {
     bool write = true;
     int before = -1;               // >= 0: this stream step runs on the stream right before the layer
     int pass = 0;                  // handed to that stream step
+    int after = -1;                // >= 0: this stream step runs on the stream right behind the layer
+    int after_pass = 0;            // handed to that one
 };
 
 // A decoder-only model: the embedding (with the position encoding's table, if it has one), the calls

@@ -1,5 +1,7 @@
-// RMS norm, the block arrangement with a norm on both sides of each sub-layer, and the clamped gated
-// feed-forward.
+// RMS norm, the block arrangements with a norm on both sides of each sub-layer and with a norm behind it only, and
+// the clamped gated feed-forward.
+#include <algorithm>
+
 #include "parts.h"
 
 namespace minillm {
@@ -138,6 +140,118 @@ private:
     int size_ = 0;               // the stream's width
 };
 
+
+// A norm BEHIND each sub-layer only; the sub-layers read the stream itself:
+//   x += norm1(mixer(x));   x += norm2(ff(x))
+// With the tensors "mixer_conv" / "ff_conv" ([width, taps] fp32) what a sub-layer reads is x + conv(x): a causal
+// convolution over time on each channel, the last tap the token's own; the last taps - 1 rows of each input are carried
+// per request in the front of the layer's state slot (the mixer's convolution first, then the feed-forward's; the
+// mixer's own state, if it has one, lies behind them). The sub-layer sets an fp32 buffer of the stream's shape and the
+// norm adds from there into the stream. Norms: [norm1] or [norm1, norm2]; parameters: dtype, size (the stream's width).
+class PostNormBlock final : public Block {
+public:
+    PostNormBlock(std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f, std::vector<std::unique_ptr<Norm>> norms, const Params& p)
+        : mixer_(std::move(m)), ff_(std::move(f)) {
+        if (!mixer_) fail("a post-norm block needs a mixer");
+        if (norms.size() != (ff_ ? 2u : 1u)) fail("a post-norm block has one norm per sub-layer (%d here), got %zu", ff_ ? 2 : 1, norms.size());
+        for (auto& n : norms) if (!n) fail("a post-norm block was handed a missing norm");
+        norm1_ = std::move(norms[0]);
+        if (ff_) norm2_ = std::move(norms[1]);
+        dtype_ = p.integer("dtype");
+        size_ = p.integer("size");
+        if (const Tensor2* c = p.weights_or_null("mixer_conv")) conv1_ = checked_conv(*c);
+        if (const Tensor2* c = p.weights_or_null("ff_conv")) {
+            if (!ff_) fail("a post-norm block without a feed-forward was handed its convolution");
+            conv2_ = checked_conv(*c);
+        }
+        conv1_bytes_ = carried_bytes(conv1_);
+        conv2_bytes_ = carried_bytes(conv2_);
+    }
+    void forward(const Tensor2& x, const StepView& step, const CacheView& cache, bool write, Arena& arena,
+                 hipStream_t s) const override {
+        const size_t carried = conv1_bytes_ + conv2_bytes_;
+        if (carried > 0 && (!cache.has_state() || cache.state_bytes < carried)) fail("a block with input convolutions needs %zu bytes of state per request", carried);
+        const size_t outer = arena.mark();
+        Tensor2 y = arena.tensor(F32, x.rows, x.cols);       // a sub-layer's result, set by it
+        const size_t mark = arena.mark();
+        CacheView rest = cache;                              // what lies behind the carried rows is the mixer's
+        if (carried > 0) {
+            rest.state = static_cast<char*>(cache.state) + carried;
+            rest.state_bytes = cache.state_bytes - carried;
+            if (rest.state_bytes == 0) rest.kind &= ~2;
+        }
+        {
+            NormedInput h(input(x, conv1_, 0, step, cache, write, arena, s));
+            mixer_->forward_set(h, step, rest, y, write, arena, s);
+        }
+        arena.release(mark);
+        norm1_->add_scaled(y, nullptr, 1.f, x, false, s);
+        StageTimes::get().mark("post_norm", s);
+        if (ff_) {
+            {
+                NormedInput h(input(x, conv2_, conv1_bytes_, step, cache, write, arena, s));
+                ff_->forward_set(h, step, y, arena, s);
+            }
+            arena.release(mark);
+            norm2_->add_scaled(y, nullptr, 1.f, x, false, s);
+            StageTimes::get().mark("post_norm2", s);
+        }
+        arena.release(outer);
+    }
+    size_t workspace_bytes(int tokens) const override {
+        size_t a = mixer_->workspace_bytes(tokens);
+        if (ff_) a = std::max(a, ff_->workspace_bytes(tokens));
+        // the sub-layer's result, and its input in the compute dtype
+        return a + static_cast<size_t>(tokens) * size_ * 8 + 2048;
+    }
+    CacheNeed cache_need() const override {
+        CacheNeed n = mixer_->cache_need();
+        if (conv1_bytes_ + conv2_bytes_ > 0) { n.kind |= 2; n.state_bytes += conv1_bytes_ + conv2_bytes_; }
+        return n;
+    }
+    void reserve(int max_seqs, hipStream_t s) const override {
+        mixer_->reserve(max_seqs, s);
+        if (ff_) ff_->reserve(max_seqs, s);
+    }
+    void add_cost(StepCost& c) const override {
+        norm1_->add_cost(c);
+        mixer_->add_cost(c);
+        if (ff_) { norm2_->add_cost(c); ff_->add_cost(c); }
+        for (const Tensor2* t : {&conv1_, &conv2_})
+            if (t->data != nullptr) { c.weight_bytes += 4.0 * t->rows * t->cols; c.flops_per_token += 2.0 * t->rows * t->cols; }
+    }
+
+private:
+    static Tensor2 checked_conv(const Tensor2& c) {
+        if (c.dtype != F32 || !c.contiguous() || c.cols < 1 || c.cols > 16) fail("a block's input convolution must be contiguous float32 [width, 1 to 16 taps]");
+        return c;
+    }
+    static size_t carried_bytes(const Tensor2& c) { return c.data ? static_cast<size_t>(c.cols - 1) * c.rows * 4 : 0; }
+    // What a sub-layer reads, in the compute dtype: x + conv(x), or x itself.
+    Tensor2 input(const Tensor2& x, const Tensor2& conv, size_t state_at, const StepView& step, const CacheView& cache, bool write,
+                  Arena& arena, hipStream_t s) const {
+        if (conv.data == nullptr) {
+            if (dtype_ != F32) fail("a post-norm block without an input convolution runs in float32 only");
+            return x;
+        }
+        if (x.cols != conv.rows) fail("the input convolution has %lld channels, the stream %lld", (long long)conv.rows, (long long)x.cols);
+        Tensor2 hc = arena.tensor(dtype_, x.rows, x.cols);
+        StateArgs st;
+        st.token_seq = step.token_seq; st.cu_q = step.cu_q; st.state_slots = step.state_slots; st.n_seqs = step.n_seqs;
+        st.max_q_len = step.max_q_len; st.state = reinterpret_cast<float*>(static_cast<char*>(cache.state) + state_at);
+        st.slot_floats = cache.slot_bytes / 4; st.n_slots = cache.n_slots; st.write = write;
+        conv_residual(x, conv, st, hc, s);
+        StageTimes::get().mark("input_conv", s);
+        return hc;
+    }
+    std::unique_ptr<Mixer> mixer_;
+    std::unique_ptr<FeedForward> ff_;
+    std::unique_ptr<Norm> norm1_, norm2_;
+    Tensor2 conv1_, conv2_;           // [width, taps], or empty: no input convolution
+    size_t conv1_bytes_ = 0, conv2_bytes_ = 0;
+    int dtype_ = BF16, size_ = 0;     // size: the stream's width
+};
+
 // y = W_down( g sigmoid(alpha g) (u + 1) ) with g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit),
 // added into the stream it is handed. Parameters: limit, alpha, dtype; tensors gate.weight, up.weight,
 // down.weight ([out, in]).
@@ -192,6 +306,10 @@ void register_gated_parts() {
     register_block("sandwich_norm", [](std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f, std::vector<std::unique_ptr<Norm>> n,
                                        const Params& p) {
         return std::unique_ptr<Block>(new SandwichNormBlock(std::move(m), std::move(f), std::move(n), p));
+    });
+    register_block("post_norm", [](std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f, std::vector<std::unique_ptr<Norm>> n,
+                                   const Params& p) {
+        return std::unique_ptr<Block>(new PostNormBlock(std::move(m), std::move(f), std::move(n), p));
     });
 }
 

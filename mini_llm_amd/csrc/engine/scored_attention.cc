@@ -20,10 +20,14 @@ const float* f32_vector(const Params& p, const char* key, int64_t n) {
 //   score  scale (q . k);  softcap > 0: softcap tanh(score / softcap);  with r1, r2 (one number per head each):
 //          minus r1 ln(1 + r2 (i - j))
 //   mask   causal, within a sliding window (0 <= i - j < window) or within the chunk of `chunk` positions that holds i
-//   out    W_o (concat_heads(softmax(score) v) * sigmoid(gate)), added into the stream.
+//   weight softmax(score) over the visible keys; or, with sigmoid_weights, sigmoid(score + score_bias[head]) for every
+//          visible key on its own, not normalised over the keys
+//   out    W_o (concat_heads(sum_j weight_j v_j) * sigmoid(gate)) (+ bias), added into the stream; with gate_per_head
+//          the gate projection has one row per head instead of one per value column.
 // Query head h reads key/value head h / (heads / kv_heads). Normed and turned keys and the values live in pages.
 // Parameters: heads, kv_heads, dim, value_dim, scale, softcap, window, chunk, rot_dims, rot_base, eps, dtype,
-// values_from_keys, gated; string qk_norm; tensors in.weight, out.weight, [q.norm, k.norm], [r1, r2].
+// values_from_keys, gated, gate_per_head, sigmoid_weights; string qk_norm; tensors in.weight, out.weight, [in.bias,
+// out.bias], [q.norm, k.norm], [r1, r2], [score_bias].
 class ScoredAttention final : public Mixer {
 public:
     explicit ScoredAttention(const Params& p) {
@@ -41,6 +45,8 @@ public:
         dtype_ = p.integer("dtype");
         values_from_keys_ = p.number("values_from_keys", 0) != 0;
         gated_ = p.number("gated", 0) != 0;
+        sh_.gate_per_head = gated_ && p.number("gate_per_head", 0) != 0;
+        sh_.sigmoid_weights = p.number("sigmoid_weights", 0) != 0;
         const int H = sh_.n_heads, G = sh_.n_kv_heads, d = sh_.dim, dv = sh_.value_dim;
         if (H < 1 || G < 1 || H % G != 0 || d < 1 || dv < 1) fail("scored_attention: %d heads over %d key/value heads of %d / %d do not fit", H, G, d, dv);
         if (sh_.window < 0 || sh_.chunk < 0 || (sh_.window > 0 && sh_.chunk > 0)) fail("scored_attention: a window or a chunk, not both");
@@ -54,12 +60,16 @@ public:
         if (sh_.norm_mode == 1) { sh_.q_norm = f32_vector(p, "q.norm", d); sh_.k_norm = f32_vector(p, "k.norm", d); }
         if (sh_.norm_mode == 2) { sh_.q_norm = f32_vector(p, "q.norm", static_cast<int64_t>(H) * d); sh_.k_norm = f32_vector(p, "k.norm", static_cast<int64_t>(G) * d); }
         if (p.weights_or_null("r1") != nullptr) { sh_.r1 = f32_vector(p, "r1", H); sh_.r2 = f32_vector(p, "r2", H); }
-        in_ = Linear(p.weights("in.weight"), nullptr);
-        out_ = Linear(p.weights("out.weight"), nullptr);
+        if (p.weights_or_null("score_bias") != nullptr) {
+            if (!sh_.sigmoid_weights) fail("scored_attention: a score bias per head goes with sigmoid weights only (a softmax cancels it)");
+            sh_.score_bias = f32_vector(p, "score_bias", H);
+        }
+        in_ = Linear(p.weights("in.weight"), p.weights_or_null("in.bias"));
+        out_ = Linear(p.weights("out.weight"), p.weights_or_null("out.bias"));
         k_col_ = H * d;
         v_col_ = values_from_keys_ ? -1 : k_col_ + G * d;
         gate_col_ = k_col_ + G * d + (values_from_keys_ ? 0 : G * dv);
-        if (in_.out_features() != gate_col_ + (gated_ ? H * dv : 0) || out_.in_features() != H * dv)
+        if (in_.out_features() != gate_col_ + (gated_ ? (sh_.gate_per_head ? H : H * dv) : 0) || out_.in_features() != H * dv)
             fail("scored_attention: the projections' shapes do not fit %d heads of %d / %d over %d key/value heads", H, d, dv, G);
     }
     void forward(NormedInput& h, const StepView& step, const CacheView& cache, const Tensor2& x, bool write, Arena& arena,

@@ -303,6 +303,31 @@ Tensor2 DeviceTensors::repeat(const Tensor2& v, int times) {
     return Tensor2(base, F32, 1, static_cast<int64_t>(n) * times);
 }
 
+Tensor2 DeviceTensors::join_cols(const std::vector<Tensor2>& parts) {
+    if (parts.empty()) throw WeightsError("join_cols: nothing to join");
+    int64_t cols = 0;
+    for (const Tensor2& t : parts) {
+        if (t.dtype != parts[0].dtype || t.rows != parts[0].rows || !t.contiguous()) throw WeightsError("join_cols: the parts must be contiguous, of one dtype and height");
+        cols += t.cols;
+    }
+    const size_t esz = parts[0].esz(), row_bytes = static_cast<size_t>(cols) * esz;
+    char* base = static_cast<char*>(allocate(static_cast<size_t>(parts[0].rows) * row_bytes, false));
+    size_t at = 0;
+    for (const Tensor2& t : parts) {
+        const size_t width = static_cast<size_t>(t.cols) * esz;
+        if (width > 0 && t.rows > 0 &&
+            hipMemcpy2D(base + at, row_bytes, t.data, width, width, static_cast<size_t>(t.rows), hipMemcpyDeviceToDevice) != hipSuccess)
+            throw WeightsError("join_cols: the copy on the device failed");
+        at += width;
+    }
+    return Tensor2(base, parts[0].dtype, parts[0].rows, cols);
+}
+
+Tensor2 DeviceTensors::zeros(int64_t n) {
+    if (n < 0) throw WeightsError("zeros: a negative size");
+    return Tensor2(allocate(static_cast<size_t>(n) * 4, true), F32, 1, n);
+}
+
 void* DeviceTensors::allocate(size_t bytes, bool zero) {
     void* p = nullptr;
     hipError_t e = hipMalloc(&p, std::max<size_t>(bytes, 16));
@@ -363,7 +388,10 @@ std::map<std::string, std::string> check_checkpoint(const std::vector<ParamSpec>
             auto it = available.find(s.name);
             if (it == available.end()) { missing.push_back(s.name); continue; }
             const std::vector<int64_t>* shape = source.shape_of(it->second);
-            if (shape == nullptr || *shape != s.shape)
+            bool fits = shape != nullptr && shape->size() == s.shape.size();
+            for (size_t k = 0; fits && k < s.shape.size(); ++k)
+                fits = static_cast<int>(k) == s.free_dim ? (*shape)[k] >= 1 : (*shape)[k] == s.shape[k];
+            if (!fits)
                 wrong.push_back(s.name + ": expected " + shape_text(s.shape) + ", found " + (shape ? shape_text(*shape) : "nothing"));
         }
         for (const auto& kv : available)
@@ -396,9 +424,13 @@ std::map<std::string, Tensor2> load_tensors(const std::vector<ParamSpec>& specs,
     for (const auto& s : specs) {
         source.read(s, source.generates() ? s.name : available.at(s.name), values);
         int64_t rows = 1, cols = 1;
-        if (s.shape.size() == 1) cols = s.shape[0];
-        else if (s.shape.size() == 2) { rows = s.shape[0]; cols = s.shape[1]; }
-        else throw WeightsError(where + ": tensor '" + s.name + "' has " + std::to_string(s.shape.size()) + " dimensions; one or two are expected");
+        // (a dimension that the checkpoint decides is read off the stored tensor)
+        std::vector<int64_t> shape = s.shape;
+        if (!source.generates() && s.free_dim >= 0)
+            if (const std::vector<int64_t>* stored = source.shape_of(available.at(s.name))) shape = *stored;
+        if (shape.size() == 1) cols = shape[0];
+        else if (shape.size() == 2) { rows = shape[0]; cols = shape[1]; }
+        else throw WeightsError(where + ": tensor '" + s.name + "' has " + std::to_string(shape.size()) + " dimensions; one or two are expected");
         if (s.add != 0.0)
             for (auto& v : values) v = static_cast<float>(v + s.add);
         const std::vector<float>* src = &values;

@@ -93,6 +93,8 @@ struct ParamSpec {
     bool transpose = false;              // stored [in, out], used as [out, in]
     double mean = 0.0, std = 0.02;
     double add = 0.0;                    // added to every value while loading (a weight stored around zero and used as 1 + w)
+    int free_dim = -1;                   // >= 0: the checkpoint decides this dimension's size (any size from 1 on; `shape` holds
+                                         // the size that the random-weights mode writes)
 };
 
 // Where tensors come from: a checkpoint on disk or the random generator. Gives fp32 host values.
@@ -151,6 +153,11 @@ public:
     Tensor2 join_rows(const std::vector<Tensor2>& parts);
     // A vector `times` times in a row ([1, times * n] fp32, a copy on the device).
     Tensor2 repeat(const Tensor2& vector, int times);
+    // Matrices of one height and dtype side by side ([rows, sum of cols], a copy on the device): several linear maps
+    // whose results are added, as one product over their inputs side by side.
+    Tensor2 join_cols(const std::vector<Tensor2>& parts);
+    // n zeros ([1, n] fp32).
+    Tensor2 zeros(int64_t n);
     size_t bytes() const { return bytes_; }
 
 private:

@@ -4,7 +4,7 @@
 #include "common.h"
 
 // ---------------------------------------------------------------------------
-// Token + position embedding: x[t,:] = wte[ids[t],:] + wpe[pos[t],:]   (fp32 out)
+// Token + position embedding: x[t,:] = scale * wte[ids[t],:] + wpe[pos[t],:]   (fp32 out)
 // /root/reference/src/kernels/embedding.cu:23-43. wpe may be null (no learned positions).
 // With `src` (optional): where src[t] >= 0, token t's id is prev[src[t]], a token that an earlier step
 // sampled on the device and the host has not read yet; ids[t] is not read then.
@@ -13,7 +13,7 @@ template <typename T>
 __global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict__ pos,
                              const T* __restrict__ wte, const T* __restrict__ wpe,
                              float* __restrict__ x, int D, const int* __restrict__ src,
-                             const int* __restrict__ prev, int n_prev) {
+                             const int* __restrict__ prev, int n_prev, float scale) {
     const int t = blockIdx.x;
     int id = ids[t];
     if (src != nullptr) {
@@ -24,9 +24,9 @@ __global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict_
     float* xr = x + static_cast<size_t>(t) * D;
     if (wpe != nullptr) {
         const T* pe = wpe + static_cast<size_t>(pos[t]) * D;
-        for (int d = threadIdx.x; d < D; d += blockDim.x) xr[d] = to_float(te[d]) + to_float(pe[d]);
+        for (int d = threadIdx.x; d < D; d += blockDim.x) xr[d] = to_float(te[d]) * scale + to_float(pe[d]);
     } else {
-        for (int d = threadIdx.x; d < D; d += blockDim.x) xr[d] = to_float(te[d]);
+        for (int d = threadIdx.x; d < D; d += blockDim.x) xr[d] = to_float(te[d]) * scale;
     }
 }
 
@@ -202,6 +202,30 @@ __global__ void reset_state_kernel(uint32_t* __restrict__ state, size_t words, c
         row[i] = 0u;
 }
 
+
+// ---------------------------------------------------------------------------
+// A weighted sum over the streams kept so far: kept holds `n_old` arrays of x's size, `stride` floats apart; x is
+// the newest. x's values are stored as array n_old of kept, and x <- sum_(j < n_old) w[j] kept_j + w[n_old] x.
+// The sum runs in the order of j (fp32).
+// ---------------------------------------------------------------------------
+#define DEPTH_MIX_MAX 64
+__global__ void depth_mix_kernel(float4* __restrict__ x, float4* __restrict__ kept, size_t stride4, int n_old,
+                                 const float* __restrict__ w, size_t n4) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n4) return;
+    const float4 newest = x[i];
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int j = 0; j < n_old; ++j) {
+        const float4 v = kept[j * stride4 + i];
+        const float a = w[j];
+        acc.x = fmaf(a, v.x, acc.x); acc.y = fmaf(a, v.y, acc.y); acc.z = fmaf(a, v.z, acc.z); acc.w = fmaf(a, v.w, acc.w);
+    }
+    const float a = w[n_old];
+    acc.x = fmaf(a, newest.x, acc.x); acc.y = fmaf(a, newest.y, acc.y); acc.z = fmaf(a, newest.z, acc.z); acc.w = fmaf(a, newest.w, acc.w);
+    kept[n_old * stride4 + i] = newest;
+    x[i] = acc;
+}
+
 extern "C" {
 
 int mllm_reset_state(void* state, size_t slot_bytes, int n_slots, const int* slots, const int* starts, int B,
@@ -216,12 +240,23 @@ int mllm_reset_state(void* state, size_t slot_bytes, int n_slots, const int* slo
 }
 
 int mllm_embed(const int* ids, const int* pos, const void* wte, const void* wpe, float* x, int T, int D,
-               int dtype, const int* src, const int* prev, int n_prev, hipStream_t stream) {
+               int dtype, const int* src, const int* prev, int n_prev, hipStream_t stream, float scale) {
     if (T <= 0) return 0;
     if (dtype == MLLM_F32)
-        embed_kernel<float><<<T, 256, 0, stream>>>(ids, pos, (const float*)wte, (const float*)wpe, x, D, src, prev, n_prev);
+        embed_kernel<float><<<T, 256, 0, stream>>>(ids, pos, (const float*)wte, (const float*)wpe, x, D, src, prev, n_prev, scale);
     else
-        embed_kernel<bf16_t><<<T, 256, 0, stream>>>(ids, pos, (const bf16_t*)wte, (const bf16_t*)wpe, x, D, src, prev, n_prev);
+        embed_kernel<bf16_t><<<T, 256, 0, stream>>>(ids, pos, (const bf16_t*)wte, (const bf16_t*)wpe, x, D, src, prev, n_prev, scale);
+    MLLM_LAUNCH_CHECK();
+    return 0;
+}
+
+// x [n floats, a multiple of 4, 16-byte aligned] and `kept` (arrays `stride` floats apart, a multiple of 4) as the
+// kernel above says; w holds n_old + 1 weights. -1: sizes that are no multiples of 4.
+int mllm_depth_mix(float* x, float* kept, size_t stride, int n_old, const float* w, size_t n, hipStream_t stream) {
+    if (n == 0) return 0;
+    if (n % 4 != 0 || stride % 4 != 0 || n_old < 0 || ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(kept)) & 15) != 0) return -1;
+    depth_mix_kernel<<<static_cast<int>((n / 4 + 255) / 256), 256, 0, stream>>>(reinterpret_cast<float4*>(x), reinterpret_cast<float4*>(kept),
+                                                                               stride / 4, n_old, w, n / 4);
     MLLM_LAUNCH_CHECK();
     return 0;
 }

@@ -62,6 +62,59 @@ rmsnorm_kernel(const float* __restrict__ x, int ldx, const int* __restrict__ row
     }
 }
 
+
+// One wavefront per (row, group): y[r, g*Dg + i] = v_i / sqrt(mean_i(v_i^2) + eps) * w[g*Dg + i] * silu(gate[r, g*Dg + i]),
+// the gate BEHIND the norm (w may be null: no weight). v is the sum of `parts` arrays part_stride floats apart, added
+// in the order of their index. The heads of a linear-attention mixer, normed one by one and gated.
+template <typename OutT, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES)
+rmsnorm_gate_after_kernel(const float* __restrict__ x, int ldx, const float* __restrict__ w, const float* __restrict__ gate, int ldg,
+                          OutT* __restrict__ y, int ldy, int n, int D, int groups, float eps, int parts, size_t part_stride) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MLLM_WAVE), lane = threadIdx.x % MLLM_WAVE;
+    const long long pair = static_cast<long long>(blockIdx.x) * WAVES + wave;
+    if (pair >= static_cast<long long>(n) * groups) return;
+    const int r = static_cast<int>(pair / groups), g = static_cast<int>(pair % groups), Dg = D / groups;
+    const float* xr = x + static_cast<size_t>(r) * ldx + g * Dg;
+    const float* gr = gate + static_cast<size_t>(r) * ldg + g * Dg;
+    OutT* yr = y + static_cast<size_t>(r) * ldy + g * Dg;
+    // up to 4 elements a lane stay in registers (heads of up to 256 columns); longer groups are read again
+    float v[4], z[4], ww[4];
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int i = min(lane + 64 * u, Dg - 1);
+        float a = xr[i];
+        for (int part = 1; part < parts; ++part) a += xr[part * part_stride + i];
+        v[u] = a;
+        z[u] = gr[i];
+        ww[u] = w ? w[g * Dg + i] : 1.f;
+        if (lane + 64 * u < Dg) ss += a * a;
+    }
+    for (int i = lane + 256; i < Dg; i += 64) {
+        float a = xr[i];
+        for (int part = 1; part < parts; ++part) a += xr[part * part_stride + i];
+        ss += a * a;
+    }
+    const float inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(Dg) + eps);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int i = lane + 64 * u;
+        if (i < Dg) yr[i] = from_float<OutT>(v[u] * inv * ww[u] * (z[u] * sigmoid_precise(z[u])));
+    }
+    for (int i = lane + 256; i < Dg; i += 64) {
+        float a = xr[i];
+        for (int part = 1; part < parts; ++part) a += xr[part * part_stride + i];
+        const float zz = gr[i];
+        yr[i] = from_float<OutT>(a * inv * (w ? w[g * Dg + i] : 1.f) * (zz * sigmoid_precise(zz)));
+    }
+}
+
+// out[i] = cap * tanh(x[i] / cap), in place (fp32)
+__global__ void softcap_kernel(float* __restrict__ x, float cap, size_t n) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) x[i] = cap * tanhf(x[i] / cap);
+}
+
 // x[r, i] += mult * scale[i] * (y[r, i] / sqrt(mean(y[r]^2) + eps) * w[i]); one wavefront per row.
 // With `clear` the row of y is set to zero behind the read, ready to collect the next sub-layer's output.
 template <int WAVES>
@@ -372,6 +425,32 @@ int mllm_rmsnorm(const float* x, int ldx, const int* rows, const float* w, const
     }
 #undef RMS
 #undef RMS_SHARES
+    MLLM_LAUNCH_CHECK();
+    return 0;
+}
+
+// y = rmsnorm(x) * w * silu(gate) in `groups` equal parts of the D columns, the gate behind the norm; w ([D]) may be
+// null. x and gate fp32 with row strides ldx / ldg; with parts > 1, x is the sum of `parts` arrays part_stride floats
+// apart. -1: D is no multiple of groups.
+int mllm_rmsnorm_gate_after(const float* x, int ldx, const float* w, const float* gate, int ldg, void* y, int ldy, int n, int D, int groups,
+                            float eps, int out_dtype, int parts, size_t part_stride, hipStream_t stream) {
+    if (n <= 0 || D <= 0) return 0;
+    if (groups < 1 || D % groups != 0 || parts < 1 || gate == nullptr) return -1;
+    const long long pairs = static_cast<long long>(n) * groups;
+    const int blocks = static_cast<int>((pairs + 3) / 4);
+    if (out_dtype == MLLM_F32)
+        rmsnorm_gate_after_kernel<float, 4><<<blocks, 256, 0, stream>>>(x, ldx, w, gate, ldg, static_cast<float*>(y), ldy, n, D, groups, eps, parts, part_stride);
+    else
+        rmsnorm_gate_after_kernel<bf16_t, 4><<<blocks, 256, 0, stream>>>(x, ldx, w, gate, ldg, static_cast<bf16_t*>(y), ldy, n, D, groups, eps, parts, part_stride);
+    MLLM_LAUNCH_CHECK();
+    return 0;
+}
+
+// x <- cap tanh(x / cap) over n contiguous floats. -1: a cap that is not positive.
+int mllm_softcap(float* x, size_t n, float cap, hipStream_t stream) {
+    if (n == 0) return 0;
+    if (!(cap > 0.f)) return -1;
+    softcap_kernel<<<static_cast<int>((n + 255) / 256), 256, 0, stream>>>(x, cap, n);
     MLLM_LAUNCH_CHECK();
     return 0;
 }

@@ -175,6 +175,9 @@ struct ScoreShape {
     int window, chunk;               // at most one of them > 0
     const float* r1;                 // per head, or null: no distance bias
     const float* r2;
+    int sigmoid;                     // != 0: a key's weight is sigmoid(score + score_bias[h]), not normalised over the keys
+    const float* score_bias;         // per head, or null
+    int gate_per_head;               // != 0: the gate has one column per head, not one per value column
 };
 
 __device__ __forceinline__ int first_visible(int p, int window, int chunk) {
@@ -216,6 +219,7 @@ scored_attention_rows(const T* __restrict__ q, int ldq, const T* __restrict__ k_
     for (int i = lane; i < d; i += 64) q_s[i] = to_float(qp[i]);
     wave_lds_sync();
     const float r1 = sh.r1 ? sh.r1[h] : 0.f, r2 = sh.r1 ? sh.r2[h] : 0.f;
+    const float pb = sh.score_bias ? sh.score_bias[h] : 0.f;
     const int kd = G * d, vd = G * dv;
     const bool vec = d % 8 == 0 && (kd * sizeof(T)) % 16 == 0 && (reinterpret_cast<uintptr_t>(k_pages) & 15) == 0;
     float m = -INFINITY, l = 0.f;
@@ -243,11 +247,18 @@ scored_attention_rows(const T* __restrict__ q, int ldq, const T* __restrict__ k_
             }
             s = shaped_score(dot, sh, r1, r2, p - j);
         }
-        const float m_new = fmaxf(m, wave_max(s));
-        const float alpha = (m == -INFINITY) ? 0.f : expf(m - m_new);
-        const float pj = valid ? expf(s - m_new) : 0.f;
-        l = l * alpha + wave_sum(pj);
-        m = m_new;
+        float alpha, pj;
+        if (sh.sigmoid) {
+            // no softmax: the weight stands for itself, nothing is rescaled or summed
+            alpha = 1.f;
+            pj = valid ? sigmoid_of(s + pb) : 0.f;
+        } else {
+            const float m_new = fmaxf(m, wave_max(s));
+            alpha = (m == -INFINITY) ? 0.f : expf(m - m_new);
+            pj = valid ? expf(s - m_new) : 0.f;
+            l = l * alpha + wave_sum(pj);
+            m = m_new;
+        }
         wave_lds_sync();          // the previous round's readers are done
         p_s[lane] = pj;
         row_s[lane] = row;
@@ -265,13 +276,13 @@ scored_attention_rows(const T* __restrict__ q, int ldq, const T* __restrict__ k_
         }
     }
     T* op = out + static_cast<size_t>(t) * ldo + h * dv;
-    const float inv_l = 1.0f / l;
+    const float inv_l = sh.sigmoid ? 1.0f : 1.0f / l;
 #pragma unroll
     for (int a = 0; a < SA_MAX_ACC; ++a) {
         const int e = lane + a * 64;
         if (e < dv) {
             float o = acc[a] * inv_l;
-            if (gate != nullptr) o *= sigmoid_of(gate[static_cast<size_t>(t) * ldg + h * dv + e]);
+            if (gate != nullptr) o *= sigmoid_of(gate[static_cast<size_t>(t) * ldg + (sh.gate_per_head ? h : h * dv + e)]);
             op[e] = from_float<T>(o);
         }
     }
@@ -341,18 +352,20 @@ int mllm_qk_prepare(const float* proj, int ld, int q_col, int k_col, int v_col, 
 }
 
 // The keys and values of the step's own tokens must be in the pages. gate (optional): fp32 [T, >= H * dv] with row
-// stride ldg; the result is multiplied by its sigmoid. -1: value rows wider than the kernel holds, heads that do
+// stride ldg (with gate_per_head: [T, >= H]); the result is multiplied by its sigmoid. With sigmoid_weights a key's
+// weight is sigmoid(score + score_bias[h]) and there is no softmax. -1: value rows wider than the kernel holds, heads that do
 // not group, a window and a chunk at once.
 int mllm_scored_attention_rows(const void* q, int ldq, const void* k_pages, const void* v_pages, const int* block_tables,
                                int max_blocks, const int* token_seq, const int* positions, int n_tokens, int H, int G, int d,
                                int dv, int page_size, float scale, float softcap, int window, int chunk, const float* r1,
-                               const float* r2, const float* gate, int ldg, void* out, int ldo, int dtype, hipStream_t stream) {
+                               const float* r2, const float* gate, int ldg, void* out, int ldo, int dtype, hipStream_t stream,
+                               int sigmoid_weights, const float* score_bias, int gate_per_head) {
     if (n_tokens <= 0) return 0;
     if (H < 1 || G < 1 || H % G != 0 || d < 1 || dv < 1 || dv > 64 * SA_MAX_ACC || page_size < 1) return -1;
     if ((window > 0 && chunk > 0) || window < 0 || chunk < 0 || (r1 != nullptr) != (r2 != nullptr)) return -1;
     const size_t smem = static_cast<size_t>(SA_WAVES) * (d + 128) * sizeof(float);
     if (smem > 60 * 1024) return -1;
-    const ScoreShape sh{scale, softcap, window, chunk, r1, r2};
+    const ScoreShape sh{scale, softcap, window, chunk, r1, r2, sigmoid_weights, score_bias, gate_per_head};
     const int blocks = (n_tokens * H + SA_WAVES - 1) / SA_WAVES;
     if (dtype == MLLM_F32)
         scored_attention_rows<float><<<blocks, SA_WAVES * 64, smem, stream>>>(
