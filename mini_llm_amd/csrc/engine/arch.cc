@@ -158,6 +158,7 @@ std::string describe_config(const Json& config) {
         t.set("shape", Json::array_of(shape));
         t.set("role", Json::of(sp.role == ParamSpec::Matrix ? "matrix" : "vector"));
         t.set("transpose", Json::of(sp.transpose));
+        if (sp.free_dim >= 0) t.set("free_dim", Json::of(static_cast<int64_t>(sp.free_dim)));
         t.set("mean", Json::of(sp.mean));
         t.set("std", Json::of(sp.std));
         tensors.push_back(t);

@@ -226,6 +226,19 @@ __global__ void depth_mix_kernel(float4* __restrict__ x, float4* __restrict__ ke
     x[i] = acc;
 }
 
+// The same one float at a time, for sizes that are no multiples of 4.
+__global__ void depth_mix_scalar_kernel(float* __restrict__ x, float* __restrict__ kept, size_t stride, int n_old,
+                                        const float* __restrict__ w, size_t n) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float newest = x[i];
+    float acc = 0.f;
+    for (int j = 0; j < n_old; ++j) acc = fmaf(w[j], kept[j * stride + i], acc);
+    acc = fmaf(w[n_old], newest, acc);
+    kept[n_old * stride + i] = newest;
+    x[i] = acc;
+}
+
 extern "C" {
 
 int mllm_reset_state(void* state, size_t slot_bytes, int n_slots, const int* slots, const int* starts, int B,
@@ -250,11 +263,16 @@ int mllm_embed(const int* ids, const int* pos, const void* wte, const void* wpe,
     return 0;
 }
 
-// x [n floats, a multiple of 4, 16-byte aligned] and `kept` (arrays `stride` floats apart, a multiple of 4) as the
-// kernel above says; w holds n_old + 1 weights. -1: sizes that are no multiples of 4.
+// x [n floats] and `kept` (arrays `stride` floats apart) as the kernels above say; w holds n_old + 1 weights.
+// Sizes that are multiples of 4 at 16-byte aligned places go four floats a thread.
 int mllm_depth_mix(float* x, float* kept, size_t stride, int n_old, const float* w, size_t n, hipStream_t stream) {
     if (n == 0) return 0;
-    if (n % 4 != 0 || stride % 4 != 0 || n_old < 0 || ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(kept)) & 15) != 0) return -1;
+    if (n_old < 0) return -1;
+    if (n % 4 != 0 || stride % 4 != 0 || ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(kept)) & 15) != 0) {
+        depth_mix_scalar_kernel<<<static_cast<int>((n + 255) / 256), 256, 0, stream>>>(x, kept, stride, n_old, w, n);
+        MLLM_LAUNCH_CHECK();
+        return 0;
+    }
     depth_mix_kernel<<<static_cast<int>((n / 4 + 255) / 256), 256, 0, stream>>>(reinterpret_cast<float4*>(x), reinterpret_cast<float4*>(kept),
                                                                                stride / 4, n_old, w, n / 4);
     MLLM_LAUNCH_CHECK();

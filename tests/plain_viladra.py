@@ -95,8 +95,9 @@ def retention_mixer(h, w, pre, m, eps):
     q = (h @ w[pre + "q"].T).view(T, H, d)
     k = (h @ w[pre + "k"].T).view(T, H, d)
     v = (h @ w[pre + "v"].T).view(T, H, e)
-    q = turn_half_split(q, pos, m["rot"]["base"], m["rot"]["dims"])
-    k = turn_half_split(k, pos, m["rot"]["base"], m["rot"]["dims"]) * d ** -0.5
+    rot = m.get("rot") or {"base": 1.0, "dims": 0}
+    q = turn_half_split(q, pos, rot["base"], rot["dims"])
+    k = turn_half_split(k, pos, rot["base"], rot["dims"]) * d ** -0.5
     decay = torch.tensor(m["decay"], dtype=h.dtype)[None, :, None].expand(T, H, d)
     o = unit_rms(decayed_outer_sums(q, k, v, decay), eps).reshape(T, H * e)
     return (o * silu(h @ w[pre + "g"].T)) @ w[pre + "o"].T
@@ -173,8 +174,9 @@ def chosen_experts(h, w, pre, mlp):
 MIXERS = {"retention": retention_mixer, "gla": gla_mixer, "attention": sigmoid_attention_mixer}
 
 
-def layer(x, w, i, lc, cfg):
-    """x + norm1(mixer(x + conv1(x))), then the same with the feed-forward, if the layer has one."""
+def layer(x, w, i, lc, cfg, gaps=None):
+    """x + norm1(mixer(x + conv1(x))), then the same with the feed-forward, if the layer has one. `gaps` (a list)
+    collects, per layer with experts, how far each token's last chosen score lies above the first one left out."""
     eps = cfg["norm"]["eps"]
     L = "l%d." % i
     canon = cfg.get("canon") is not None
@@ -182,18 +184,20 @@ def layer(x, w, i, lc, cfg):
     x = x + unit_rms(MIXERS[lc["type"]](h, w, L + "mix.", lc["mixer"], eps), eps) * w[L + "norm1"]
     if lc.get("mlp") is not None:
         h = input_convolution(x, w[L + "canon2"]) if canon else x
+        if gaps is not None:
+            gaps.append(chosen_experts(h, w, L + "mlp.", lc["mlp"])[1])
         x = x + unit_rms(routed_experts(h, w, L + "mlp.", lc["mlp"]), eps) * w[L + "norm2"]
     return x
 
 
-def streams(cfg, w, tokens: List[int]):
+def streams(cfg, w, tokens: List[int], gaps=None):
     """The residual stream as every layer hands it on ([layers, T, D]) and the last one. What layer i hands on is
     sum_j dwa_i[j] X_j over X_0 (the embedding's output) and the results X_1 .. X_(i+1) of the layers so far."""
     x = w["embed"][torch.tensor(tokens)] * cfg["embedding"]["scale"]
     kept = [x]
     handed = []
     for i, lc in enumerate(cfg["layers"]):
-        kept.append(layer(x, w, i, lc, cfg))
+        kept.append(layer(x, w, i, lc, cfg, gaps))
         a = w["l%d.dwa" % i]
         x = sum(a[j] * kept[j] for j in range(i + 2))
         handed.append(x)
@@ -206,3 +210,28 @@ def logits(cfg, w, tokens: List[int]):
     z = (unit_rms(x, cfg["norm"]["eps"]) * w["final.norm"]) @ w["embed"].T
     cap = cfg.get("logit_softcap")
     return cap * torch.tanh(z / cap) if cap else z
+
+
+def forward(cfg, w, tokens: List[int]):
+    return logits(cfg, w, tokens)
+
+
+def closest_call(cfg, w, tokens: List[int]):
+    """[T]: per token, the smallest gap over the layers between the last chosen expert's score and the first one
+    left out (1 where no layer has a choice to make). A token with a small gap is one whose experts a rounding can change."""
+    gaps: List[torch.Tensor] = []
+    streams(cfg, w, tokens, gaps)
+    out = torch.ones(len(tokens), dtype=torch.float64)
+    for g in gaps:
+        out = torch.minimum(out, g)
+    return out
+
+
+def greedy_generate(cfg, w, prompt: List[int], n_new: int) -> List[int]:
+    """n_new tokens, each the largest logit's (the lowest index on a tie) given everything before it."""
+    ids, out = list(prompt), []
+    for _ in range(n_new):
+        nxt = int(torch.argmax(logits(cfg, w, ids)[-1]))
+        out.append(nxt)
+        ids.append(nxt)
+    return out

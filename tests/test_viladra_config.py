@@ -1,0 +1,154 @@
+"""Viladra without a GPU: what its configuration asks of a checkpoint, what it refuses, and the plain
+implementation's own consistency (the recurrence carried over a cut, the window's edges, the experts' choice, the
+weighted sum over the layers)."""
+import copy
+
+import pytest
+import torch
+
+import plain_viladra as pv
+import viladra_cases as vc
+from mini_llm_amd import check_model_dir, describe_config, registered_architectures, write_random_model
+from mini_llm_amd.config import ConfigError
+from mini_llm_amd.weights import WeightsError
+
+
+def test_registered_and_tensors_follow_the_layer_list():
+    assert "Viladra" in registered_architectures()
+    d = describe_config(vc.MIXED_A)
+    assert d["architecture"] == "Viladra"
+    shapes = {t["name"]: t["shape"] for t in d["tensors"]}
+    assert shapes["embed"] == [257, 64] and "head" not in shapes and shapes["final.norm"] == [64]
+    # gla: queries and keys heads * dim, values and gate heads * vdim, the decays' low-rank map, one norm weight for all heads
+    assert shapes["l0.mix.q"] == [32, 64] and shapes["l0.mix.v"] == [32, 64] and shapes["l0.mix.norm"] == [16]
+    assert shapes["l4.mix.a1"] == [3, 64] and shapes["l4.mix.a2"] == [32, 3] and shapes["l4.mix.a2.b"] == [32]
+    # attention: grouped keys and values of a width of their own, norms over the whole projections, one gate row per head
+    assert shapes["l1.mix.q"] == [64, 64] and shapes["l1.mix.k"] == [32, 64] and shapes["l1.mix.v"] == [48, 64]
+    assert shapes["l1.mix.q.norm"] == [64] and shapes["l1.mix.k.norm"] == [32] and shapes["l1.mix.pb"] == [4] and shapes["l1.mix.g"] == [4, 64]
+    assert shapes["l1.mix.o"] == [64, 96] and shapes["l1.mix.o.b"] == [64] and shapes["l1.mix.v.b"] == [48]
+    # retention: no norm weight, no biases
+    assert shapes["l2.mix.g"] == [96, 64] and shapes["l2.mix.o"] == [64, 96] and "l2.mix.norm" not in shapes and "l2.mix.q.b" not in shapes
+    # experts one by one, the router, the shared expert where there is one; a layer without a feed-forward has none of them
+    assert shapes["l1.mlp.e5.up"] == [16, 64] and shapes["l1.mlp.e5.down"] == [64, 16] and "l1.mlp.e6.up" not in shapes
+    assert shapes["l1.mlp.router"] == [6, 64] and shapes["l1.mlp.shared.up"] == [24, 64] and "l3.mlp.shared.up" not in shapes
+    assert "l2.norm2" not in shapes and "l2.canon2" not in shapes and "l2.mlp.router" not in shapes and shapes["l2.canon1"] == [64, 3]
+    # the weights of the sum over the layers: one more per layer
+    assert [shapes["l%d.dwa" % i] for i in range(5)] == [[2], [3], [4], [5], [6]]
+    roles = {t["name"]: t["role"] for t in d["tensors"]}
+    assert roles["l0.mlp.router"] == "vector" and roles["l0.mix.a2"] == "vector" and roles["l0.mix.a1"] == "matrix" and roles["l0.dwa"] == "vector"
+    free = {t["name"]: t.get("free_dim") for t in d["tensors"]}
+    assert free["l0.mix.a1"] == 0 and free["l0.mix.a2"] == 1 and free["l0.mix.q"] is None
+
+
+@pytest.mark.parametrize("change, message", [
+    (lambda c: c["layers"][1].__setitem__("type", "lstm"), "unknown layer type"),
+    (lambda c: c["layers"][1]["mixer"].__setitem__("kv_heads", 3), "multiple of kv_heads"),
+    (lambda c: c["layers"][2]["mixer"]["rot"].__setitem__("dims", 3), "even"),
+    (lambda c: c["layers"][2]["mixer"]["rot"].__setitem__("dims", 10), "at most dim"),
+    (lambda c: c["layers"][2]["mixer"].__setitem__("decay", [0.5]), "one number per head"),
+    (lambda c: c["layers"][2]["mixer"].__setitem__("decay", [0.5, 0.5, 1.5, 0.5]), "(0, 1]"),
+    (lambda c: c["layers"][0]["mixer"].__setitem__("tau", 0.0), "tau"),
+    (lambda c: c["layers"][0]["mlp"].__setitem__("kind", "dense"), "moe"),
+    (lambda c: c["layers"][0]["mlp"]["router"].__setitem__("top", 9), "top"),
+    (lambda c: c["layers"][1]["mixer"].pop("mask"), "mask"),
+    (lambda c: c["canon"].__setitem__("taps", 17), "16 taps"),
+    (lambda c: c.__setitem__("logit_softcap", -1.0), "logit_softcap"),
+    (lambda c: c.pop("norm"), "norm"),
+])
+def test_refusals(change, message):
+    cfg = copy.deepcopy(vc.MIXED_A)
+    change(cfg)
+    with pytest.raises(ConfigError, match=message.replace("(", r"\(").replace("]", r"\]")):
+        describe_config(cfg)
+
+
+def test_written_folder_checks_a_missing_tensor_is_named_and_the_rank_is_the_checkpoints(tmp_path):
+    d = write_random_model(dict(vc.MIXED_B), str(tmp_path / "m"), 1)
+    arch, n_tensors, _ = check_model_dir(d)
+    assert arch == "Viladra" and n_tensors == len(describe_config(vc.MIXED_B)["tensors"])
+    from safetensors.torch import load_file, save_file
+    t = load_file(str(tmp_path / "m" / "model.safetensors"))
+    del t["l1.mlp.e7.down"]
+    save_file(t, str(tmp_path / "m" / "model.safetensors"))
+    with pytest.raises(WeightsError, match="l1.mlp.e7.down"):
+        check_model_dir(d)
+    # a low-rank map of another rank than the configuration would write is taken as stored; a height that is wrong is not
+    d2 = write_random_model(dict(vc.ONLY_GLA), str(tmp_path / "g"), 1)
+    t = load_file(str(tmp_path / "g" / "model.safetensors"))
+    t["l0.mix.a1"] = torch.randn(9, t["l0.mix.a1"].shape[1]).to(t["l0.mix.a1"].dtype)
+    t["l0.mix.a2"] = torch.randn(t["l0.mix.a2"].shape[0], 9).to(t["l0.mix.a2"].dtype)
+    save_file(t, str(tmp_path / "g" / "model.safetensors"))
+    assert check_model_dir(d2)[0] == "Viladra"
+    t["l0.mix.a2"] = torch.randn(5, 9).to(t["l0.mix.a2"].dtype)
+    save_file(t, str(tmp_path / "g" / "model.safetensors"))
+    with pytest.raises(WeightsError, match="l0.mix.a2"):
+        check_model_dir(d2)
+
+
+def test_plain_recurrence_carried_over_a_cut_and_its_closed_form():
+    """The recurrence over a sequence equals the weighted sum it stands for: o_t = sum_(s <= t) (prod_(s < r <= t) f_r
+    * k_s) . q_t v_s; with decay 1 it is the plain sum over all earlier tokens."""
+    g = torch.Generator().manual_seed(0)
+    T, H, d, e = 9, 2, 3, 4
+    q, k = torch.randn(T, H, d, generator=g, dtype=torch.float64), torch.randn(T, H, d, generator=g, dtype=torch.float64)
+    v = torch.randn(T, H, e, generator=g, dtype=torch.float64)
+    f = torch.rand(T, H, d, generator=g, dtype=torch.float64)
+    o = pv.decayed_outer_sums(q, k, v, f)
+    for t in (0, 4, 8):
+        for h in range(H):
+            ref = torch.zeros(e, dtype=torch.float64)
+            for s in range(t + 1):
+                ref += ((f[s + 1:t + 1, h].prod(0) * k[s, h]) @ q[t, h]) * v[s, h]
+            assert torch.allclose(o[t, h], ref, atol=1e-12)
+    ones = pv.decayed_outer_sums(q, k, v, torch.ones_like(f))
+    assert torch.allclose(ones[5, 1], sum((k[s, 1] @ q[5, 1]) * v[s, 1] for s in range(6)), atol=1e-12)
+
+
+def test_plain_window_edges_and_weights_without_a_softmax(tmp_path):
+    """A key just inside the window counts, the one just outside does not; doubling one value row changes only
+    the rows that see it, by exactly that key's weight times the row (the weights are not normalised)."""
+    d = write_random_model(dict(vc.ONLY_ATTENTION), str(tmp_path / "m"), 2)
+    cfg, w = pv.read_model(d)
+    m, eps, W = cfg["layers"][0]["mixer"], cfg["norm"]["eps"], cfg["layers"][0]["mixer"]["mask"]["size"]
+    g = torch.Generator().manual_seed(1)
+    h = torch.randn(30, cfg["width"], generator=g, dtype=torch.float64)
+    a = pv.sigmoid_attention_mixer(h, w, "l0.mix.", m, eps)
+    h2 = h.clone()
+    h2[10] += 1.0
+    b = pv.sigmoid_attention_mixer(h2, w, "l0.mix.", m, eps)
+    changed = [(a[t] - b[t]).abs().max() > 1e-9 for t in range(30)]
+    assert changed == [10 <= t < 10 + W for t in range(30)]
+
+
+def test_plain_experts_choice_and_weights(tmp_path):
+    d = write_random_model(dict(vc.ONLY_EXPERTS), str(tmp_path / "m"), 3)
+    cfg, w = pv.read_model(d)
+    mlp = cfg["layers"][0]["mlp"]
+    g = torch.Generator().manual_seed(2)
+    h = torch.randn(11, cfg["width"], generator=g, dtype=torch.float64)
+    out = pv.routed_experts(h, w, "l0.mlp.", mlp)
+    chosen, _ = pv.chosen_experts(h, w, "l0.mlp.", mlp)
+    scores = torch.softmax(h @ w["l0.mlp.router"].T, -1)
+    for t in range(11):
+        ref = pv.small_ff(h[t:t + 1], w, "l0.mlp.shared.")[0]
+        for x in chosen[t].tolist():
+            ref = ref + mlp["router"]["scale"] * scores[t, x] * pv.small_ff(h[t:t + 1], w, "l0.mlp.e%d." % x)[0]
+        assert torch.allclose(out[t], ref, atol=1e-12)
+    assert chosen.shape == (11, mlp["router"]["top"])
+
+
+def test_plain_prompt_equals_its_prefixes_and_the_sum_over_the_layers(tmp_path):
+    """Logits of a prefix do not depend on what follows; what the last layer hands on is the weighted sum of the
+    embedding's output and every layer's result."""
+    d = write_random_model(dict(vc.MIXED_A), str(tmp_path / "m"), 4)
+    cfg, w = pv.read_model(d)
+    toks = vc.requests(cfg["vocab"], [17], seed=3)["r0"]
+    full = pv.forward(cfg, w, toks)
+    for n in (1, 5, 12):
+        assert torch.allclose(pv.forward(cfg, w, toks[:n]), full[:n], atol=1e-10)
+    handed, last = pv.streams(cfg, w, toks)
+    x = w["embed"][torch.tensor(toks)] * cfg["embedding"]["scale"]
+    kept = [x]
+    for i, lc in enumerate(cfg["layers"]):
+        kept.append(pv.layer(x if i == 0 else handed[i - 1], w, i, lc, cfg))
+        assert torch.allclose(handed[i], sum(w["l%d.dwa" % i][j] * kept[j] for j in range(i + 2)), atol=1e-12)
