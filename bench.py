@@ -86,7 +86,34 @@ def rekirax_config(n_layer, size="gpt2-small", n_positions=1024):
             "vocab_size": 50257, "n_positions": n_positions, "n_layer": n + 3}
 
 
-DESIGNS = {"kugulorn": kugulorn_config, "rekirax": rekirax_config}
+def viladra_config(n_layer, size="gpt2-small", n_positions=1024):
+    """A Viladra model with as many layers as the GPT-2 configuration `size` has, at the same width, vocabulary and
+    context: linear attention with a decay per key channel (gla), retention and windowed sigmoid attention in turn,
+    heads of 64 as many as GPT-2 has (a quarter as many key/value heads, a window of 512, 32 rotated columns, decays'
+    maps of rank 16), four taps, each layer with eight experts of which two are chosen beside a shared one; all
+    experts together hold what GPT-2's two feed-forward matrices do (the shared one a quarter of it)."""
+    full_layers, d, h, f = SIZES[size]
+    n = n_layer or full_layers
+    kv = max(k for k in range(1, max(h // 4, 1) + 1) if h % k == 0)
+    mlp = {"kind": "moe", "router": {"experts": 8, "top": 2, "scale": 2.0}, "expert": {"ff": 3 * f // 32}, "shared": {"ff": f // 4}}
+    layers = []
+    for i in range(n):
+        if i % 3 == 0:
+            layers.append({"type": "gla", "mlp": mlp, "mixer": {"heads": h, "dim": 64, "vdim": 64, "tau": 16.0, "rank": 16}})
+        elif i % 3 == 1:
+            layers.append({"type": "retention", "mlp": mlp,
+                           "mixer": {"heads": h, "dim": 64, "vdim": 64, "decay": [1.0 - 2.0 ** -(5 + 5 * k / h) for k in range(h)],
+                                     "rot": {"base": 10000.0, "dims": 32}}})
+        else:
+            layers.append({"type": "attention", "mlp": mlp,
+                           "mixer": {"heads": h, "kv_heads": kv, "dim": 64, "vdim": 64, "scale": 0.125, "mask": {"size": 512}}})
+    return {"architecture": "Viladra", "vocab": 50257, "width": d, "norm": {"eps": 1e-6}, "canon": {"taps": 4},
+            "embedding": {"scale": 1.0}, "logit_softcap": 30.0, "layers": layers,
+            # (what the measurement itself reads; the architecture ignores them)
+            "vocab_size": 50257, "n_positions": n_positions, "n_layer": n}
+
+
+DESIGNS = {"kugulorn": kugulorn_config, "rekirax": rekirax_config, "viladra": viladra_config}
 
 
 def decode_run(model_dir, dtype, batch, prompt_len, steps, warmup, cfg):
@@ -267,10 +294,12 @@ def compare_main(args):
     """--compare: both designs at one size through prefill_run and decode_run."""
     from mini_llm_amd import Runner, write_random_model
     other = args.design if args.design in DESIGNS else "kugulorn"
-    out = {"metric": f"{other.capitalize()} beside GPT-2 at {args.size} sizes: prefill tok/s (2 x 1,024 tokens) and decode tok/s",
+    base = args.beside
+    names = {"gpt2": "GPT-2"}
+    out = {"metric": f"{other.capitalize()} beside {names.get(base, base.capitalize())} at {args.size} sizes: prefill tok/s (2 x 1,024 tokens) and decode tok/s",
            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights seed 2, uniform random token ids)",
            "n_gpus": 1, "designs": {}}
-    for design in ("gpt2", other):
+    for design in (base, other):
         cfg = (DESIGNS[design] if design in DESIGNS else small_config)(args.layers, args.size, args.positions)
         with tempfile.TemporaryDirectory() as d:
             write_random_model(dict(cfg), d, seed=2)
@@ -287,8 +316,8 @@ def compare_main(args):
                 rec[f"decode_b{b}"] = {"tok_per_s": round(tps, 1), "ms_per_step": round(step_s * 1e3, 4), "mean_context": round(mean_ctx, 1),
                                        "GBps": round(bytes_step / step_s / 1e9, 1), "frac_of_hbm_peak": round(bytes_step / step_s / HBM_PEAK, 5)}
             out["designs"][design] = rec
-    g, k = out["designs"]["gpt2"], out["designs"][other]
-    out[other + "_over_gpt2"] = {"prefill": round(k["prefill"]["tok_per_s"] / g["prefill"]["tok_per_s"], 3),
+    g, k = out["designs"][base], out["designs"][other]
+    out[other + "_over_" + base] = {"prefill": round(k["prefill"]["tok_per_s"] / g["prefill"]["tok_per_s"], 3),
                                  **{f"decode_b{b}": round(k[f"decode_b{b}"]["tok_per_s"] / g[f"decode_b{b}"]["tok_per_s"], 3) for b in (1, 8, 64)}}
     print(json.dumps(out))
     return 0
@@ -318,9 +347,11 @@ def main():
     ap.add_argument("--config", help="a config.json to measure in place of the GPT-2 sizes (any registered architecture; "
                                      "it names vocab_size and n_positions, or --vocab / --positions do)")
     ap.add_argument("--vocab", type=int, default=0, help="with --config: the vocabulary to draw token ids from")
-    ap.add_argument("--design", default="gpt2", choices=["gpt2", "kugulorn", "rekirax"],
-                    help="kugulorn / rekirax: a model of that design of about the size --size names (kugulorn_config, "
-                         "rekirax_config) through the same measurement; --compare runs it and GPT-2 one after the other")
+    ap.add_argument("--design", default="gpt2", choices=["gpt2", "kugulorn", "rekirax", "viladra"],
+                    help="kugulorn / rekirax / viladra: a model of that design of about the size --size names (kugulorn_config, "
+                         "rekirax_config, viladra_config) through the same measurement; --compare runs it and GPT-2 one after the other")
+    ap.add_argument("--beside", default="gpt2", choices=["gpt2", "kugulorn", "rekirax", "viladra"],
+                    help="with --compare: the design that the --design model is measured beside (default GPT-2)")
     ap.add_argument("--compare", action="store_true",
                     help="prefill (2 x 1,024 tokens) and decode (batch 1, 8, 64) of the --design model (default Kugulorn) and of the GPT-2 model "
                          "of --size, side by side in one JSON line")
