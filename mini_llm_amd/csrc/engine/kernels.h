@@ -147,10 +147,8 @@ int mllm_concat_cast(const float* a, const float* b, int T, int D, void* out, in
 int mllm_glu_act(const void* gu, int ld, int T, int F, int act, void* out, int ldo, int dtype, hipStream_t stream);
 
 // moe.hip
-int mllm_moe_route(const void* h, int ldh, int dtype, const float* w, int T, int D, int E, int top, float scale, float* weights, int ldw,
-                   hipStream_t stream);
-int mllm_moe_act(const void* up, int ldu, const float* weights, int ldw, int E, int ff, int shared_ff, void* out, int ldo, int T, int dtype,
-                 hipStream_t stream);
+int mllm_moe_act(const void* up, int ldu, const float* logits, int ldl, int E, int ff, int shared_ff, int top, float scale, void* out, int ldo,
+                 float* weights_out, int ldw, int T, int dtype, hipStream_t stream);
 
 // sampling.hip
 int mllm_argmax_chunks(int V);

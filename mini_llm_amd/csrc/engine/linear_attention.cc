@@ -133,12 +133,13 @@ private:
 
 // A mixture of small feed-forward experts beside an optional shared one:
 //   y = sum_(e chosen) w_e W_down,e act(W_up,e h) + W_down,s act(W_up,s h),   act(z) = relu(z)^2
-// The router's logits W_r h and their softmax over all experts are fp32; the `top` experts with the largest scores are
-// chosen (the lower index wins a tie) and w_e = scale * score_e, not renormalised. The experts' first products are one
+// The router's logits W_r h are a product of their own with fp32 results (its operands are the compute dtype's: a
+// checkpoint's bfloat16 router is held exactly), their softmax over all experts is fp32; the `top` experts with the
+// largest scores are chosen (the lower index wins a tie) and w_e = scale * score_e, not renormalised. The experts' first products are one
 // joined product (up.weight rows [expert 0 | expert 1 | ... | shared]), the activation multiplies every expert's
 // block by w_e (zero for an expert that was not chosen), and the second products are one joined product too
 // (down.weight columns in the same order).
-// Parameters: dtype, experts, ff (an expert's hidden width), top, scale; tensors router [experts, width] fp32,
+// Parameters: dtype, experts, ff (an expert's hidden width), top, scale; tensors router [experts, width],
 // up.weight [experts * ff + shared_ff, width], down.weight [width, experts * ff + shared_ff].
 class RoutedExperts final : public FeedForward {
 public:
@@ -150,10 +151,10 @@ public:
         if (act != "relu2") fail("routed_experts: unknown activation '%s' (known: relu2)", act.c_str());
         up_ = Linear(p.weights("up.weight"), nullptr);
         down_ = Linear(p.weights("down.weight"), nullptr);
-        router_ = p.weights("router");
+        router_ = Linear(p.weights("router"), nullptr);
         if (E_ < 1 || ff_ < 1 || top_ < 1 || top_ > E_) fail("routed_experts: %d of %d experts of %d do not fit", top_, E_, ff_);
-        if (router_.dtype != F32 || !router_.contiguous() || router_.rows != E_ || router_.cols != up_.in_features())
-            fail("routed_experts: the router must be contiguous float32 [%d, %d]", E_, up_.in_features());
+        if (router_.out_features() != E_ || router_.in_features() != up_.in_features())
+            fail("routed_experts: the router must be [%d, %d]", E_, up_.in_features());
         if (up_.out_features() < E_ * ff_ || down_.in_features() != up_.out_features() || down_.out_features() != up_.in_features())
             fail("routed_experts: the joined products' shapes do not fit %d experts of %d", E_, ff_);
     }
@@ -166,32 +167,31 @@ public:
     void run(NormedInput& h, const StepView& step, const Tensor2& x, Arena& arena, hipStream_t s, int out_epilogue) const {
         const int T = step.n_tokens, N = up_.out_features();
         const Tensor2& in = h.tensor(arena, s);
-        Tensor2 weights = arena.tensor(F32, T, E_);
-        moe_route(in, router_, top_, scale_, weights, s);
+        const int lde = (E_ + 3) / 4 * 4;
+        Tensor2 logits(arena.take(static_cast<size_t>(T) * lde * 4), F32, T, E_, lde);
+        router_(in, logits, STORE_F32, nullptr, s);
         StageTimes::get().mark("router", s);
         Tensor2 inner = arena.tensor(dtype_, T, N);
         up_(in, inner, STORE, nullptr, s);
         StageTimes::get().mark("fc1", s);
-        moe_act(inner, &weights, E_, ff_, inner, s);            // in place
+        moe_act(inner, logits, ff_, top_, scale_, inner, nullptr, s);            // in place
         down_(inner, x, out_epilogue, nullptr, s);
         StageTimes::get().mark("fc2", s);
     }
     size_t workspace_bytes(int tokens) const override {
-        return static_cast<size_t>(tokens) * ((up_.out_features() + up_.in_features()) * dtype_size(dtype_) + E_ * 4) + 2048;
+        return static_cast<size_t>(tokens) * ((up_.out_features() + up_.in_features()) * dtype_size(dtype_) + (E_ + 4) * 4) + 2048;
     }
     void reserve(int, hipStream_t s) const override { reserve_linear_scratch(s); }
     void add_cost(StepCost& c) const override {
         up_.add_cost(c);
         down_.add_cost(c);
-        c.weight_bytes += 4.0 * E_ * router_.cols;
-        c.flops_per_token += 2.0 * E_ * router_.cols;
+        router_.add_cost(c);
     }
 
 private:
     int dtype_ = BF16, E_ = 0, ff_ = 0, top_ = 0;
     float scale_ = 1.f;
-    Linear up_, down_;
-    Tensor2 router_;
+    Linear up_, down_, router_;
 };
 
 // What a layer hands on is a weighted sum of the embedding's output and the results of all layers so far: behind the

@@ -332,12 +332,12 @@ void softcap(const Tensor2& x, float cap, hipStream_t stream);
 void depth_mix(const Tensor2& x, const Tensor2& kept, int n_old, const float* w, hipStream_t stream);
 
 // -- mixture of experts -----------------------------------------------------------------------------
-// weights[t, e] = scale * softmax(w h_t)[e] for the `top` experts with the largest scores (the lower index wins a tie),
-// 0 for the others. h [T, D] in its dtype, w [E, D] fp32, weights [T, E] fp32.
-void moe_route(const Tensor2& h, const Tensor2& w, int top, float scale, const Tensor2& weights, hipStream_t stream);
-// out[t, e * ff + j] = weights[t, e] * relu(up[t, e * ff + j])^2 for n_experts experts of ff columns; the columns behind
-// them (a shared expert's) are relu(.)^2 alone. out may be up.
-void moe_act(const Tensor2& up, const Tensor2* weights, int n_experts, int ff, const Tensor2& out, hipStream_t stream);
+// From a token's router logits ([T, E] fp32): scores softmax(logits) over all experts, the `top` largest chosen (the
+// lower index wins a tie), weight_e = scale * score_e for them and 0 for the others. Then
+// out[t, e * ff + j] = weight_e * relu(up[t, e * ff + j])^2 for the E experts of ff columns; the columns behind them (a
+// shared expert's) are relu(.)^2 alone. out may be up. `weights` (optional, [T, E] fp32) receives the weights.
+void moe_act(const Tensor2& up, const Tensor2& logits, int ff, int top, float scale, const Tensor2& out, const Tensor2* weights,
+             hipStream_t stream);
 
 // out = [a | b] row by row in out's dtype (a, b fp32 [T, D])
 void concat_cast(const Tensor2& a, const Tensor2& b, const Tensor2& out, hipStream_t stream);

@@ -253,31 +253,24 @@ void depth_mix(const Tensor2& x, const Tensor2& kept, int n_old, const float* w,
                          static_cast<size_t>(x.rows) * x.cols, stream), "depth_mix");
 }
 
-void moe_route(const Tensor2& h, const Tensor2& w, int top, float scale, const Tensor2& weights, hipStream_t stream) {
-    need_act(h, "moe_route: h");
-    need_f32(w, "moe_route: the router");
-    need_f32(weights, "moe_route: the weights");
-    if (!w.contiguous() || w.cols != h.cols || weights.rows != h.rows || weights.cols != w.rows) fail("moe_route: the router must be [E, %lld] and the weights [%lld, E]", (long long)h.cols, (long long)h.rows);
-    if (top < 1 || top > w.rows) fail("moe_route: %d of %lld experts", top, (long long)w.rows);
-    check(mllm_moe_route(h.data, i32(h.stride), h.dtype, static_cast<const float*>(w.data), i32(h.rows), i32(h.cols), i32(w.rows), top, scale,
-                         static_cast<float*>(weights.data), i32(weights.stride), stream), "moe_route");
-}
-
-void moe_act(const Tensor2& up, const Tensor2* weights, int n_experts, int ff, const Tensor2& out, hipStream_t stream) {
+void moe_act(const Tensor2& up, const Tensor2& logits, int ff, int top, float scale, const Tensor2& out, const Tensor2* weights,
+             hipStream_t stream) {
     need_act(up, "moe_act: up");
+    need_f32(logits, "moe_act: the router's logits");
     if (out.dtype != up.dtype || out.rows != up.rows || out.cols != up.cols) fail("moe_act: out must have up's shape and dtype");
-    if (n_experts < 0 || ff < 1 || static_cast<int64_t>(n_experts) * ff > up.cols) fail("moe_act: %d experts of %d columns do not fit rows of %lld", n_experts, ff, (long long)up.cols);
-    const float* wp = nullptr;
+    const int E = i32(logits.cols);
+    if (logits.rows != up.rows || E < 1 || ff < 1 || static_cast<int64_t>(E) * ff > up.cols) fail("moe_act: %d experts of %d columns do not fit rows of %lld", E, ff, (long long)up.cols);
+    if (top < 1 || top > E) fail("moe_act: %d of %d experts", top, E);
+    float* wp = nullptr;
     int ldw = 0;
-    if (n_experts > 0) {
-        if (weights == nullptr) fail("moe_act: the experts' weights are missing");
+    if (weights != nullptr) {
         need_f32(*weights, "moe_act: the weights");
-        if (weights->rows != up.rows || weights->cols != n_experts) fail("moe_act: the weights must be [%lld, %d]", (long long)up.rows, n_experts);
-        wp = static_cast<const float*>(weights->data);
+        if (weights->rows != up.rows || weights->cols != E) fail("moe_act: the weights must be [%lld, %d]", (long long)up.rows, E);
+        wp = static_cast<float*>(weights->data);
         ldw = i32(weights->stride);
     }
-    check(mllm_moe_act(up.data, i32(up.stride), wp, ldw, n_experts, ff, i32(up.cols) - n_experts * ff, out.data, i32(out.stride), i32(up.rows), up.dtype, stream),
-          "moe_act");
+    check(mllm_moe_act(up.data, i32(up.stride), static_cast<const float*>(logits.data), i32(logits.stride), E, ff, i32(up.cols) - E * ff, top, scale,
+                       out.data, i32(out.stride), wp, ldw, i32(up.rows), up.dtype, stream), "moe_act");
 }
 
 void concat_cast(const Tensor2& a, const Tensor2& b, const Tensor2& out, hipStream_t stream) {

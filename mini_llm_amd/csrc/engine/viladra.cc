@@ -209,7 +209,7 @@ std::vector<ParamSpec> viladra_specs(const Json& config) {
                 matrix(E + "up", f.ff, D);
                 matrix(E + "down", D, f.ff);
             }
-            s.push_back({L + "mlp.router", {f.experts, D}, ParamSpec::Vector, false, 0.0, 1.0 / std::sqrt(static_cast<double>(D))});
+            matrix(L + "mlp.router", f.experts, D);
             if (f.shared_ff > 0) {
                 matrix(L + "mlp.shared.up", f.shared_ff, D);
                 matrix(L + "mlp.shared.down", D, f.shared_ff);

@@ -2,6 +2,8 @@
 //   s = scale (q . k);  softcap > 0: s <- softcap tanh(s / softcap);  r1: s <- s - r1[h] ln(1 + r2[h] (i - j));
 // and which keys a query sees besides the sliding window the kernels take on their own: with chunk > 0 only those
 // of the block of `chunk` positions (counted from 0) that holds the query.
+// With `sigmoid` the weight of a visible key is sigmoid(s + score_bias[h]) on its own, not a softmax over the keys,
+// and with `gate_per_head` the result's gate has one number per head and row, not one per output column.
 #pragma once
 
 struct MllmScoreShape {
@@ -9,4 +11,7 @@ struct MllmScoreShape {
     int chunk;               // <= 0: none
     const float* r1;         // per head, or null: no distance bias
     const float* r2;
+    int sigmoid;             // 0: softmax weights
+    const float* score_bias; // per head, or null (sigmoid weights only)
+    int gate_per_head;
 };

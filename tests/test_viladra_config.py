@@ -35,7 +35,7 @@ def test_registered_and_tensors_follow_the_layer_list():
     # the weights of the sum over the layers: one more per layer
     assert [shapes["l%d.dwa" % i] for i in range(5)] == [[2], [3], [4], [5], [6]]
     roles = {t["name"]: t["role"] for t in d["tensors"]}
-    assert roles["l0.mlp.router"] == "vector" and roles["l0.mix.a2"] == "vector" and roles["l0.mix.a1"] == "matrix" and roles["l0.dwa"] == "vector"
+    assert roles["l0.mlp.router"] == "matrix" and roles["l0.mix.a2"] == "vector" and roles["l0.mix.a1"] == "matrix" and roles["l0.dwa"] == "vector"
     free = {t["name"]: t.get("free_dim") for t in d["tensors"]}
     assert free["l0.mix.a1"] == 0 and free["l0.mix.a2"] == 1 and free["l0.mix.q"] is None
 
