@@ -402,6 +402,10 @@ bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_
                                          a.out.data, static_cast<int>(a.out.stride), a.q.dtype, stream), "scored_attention (rows)");
     };
     if (a.shape != nullptr && a.q_col != 0) fail("paged_attention: shaped scores take queries from column 0");
+    if (a.shape != nullptr && (a.shape->sigmoid || a.shape->gate_per_head) &&
+        !(a.q.dtype == BF16 && (a.head_dim == 32 || a.head_dim == 64 || a.head_dim == 128) && pow2(a.page_size) && a.page_size >= a.head_dim / 16 &&
+          a.max_blocks <= 2048 && (a.max_q_len == 1 || (a.cu_q != nullptr && a.ctx_len != nullptr))))
+        fail("paged_attention: sigmoid weights and a gate per head are taken in bfloat16 at head sizes 32, 64 and 128 only");
     const int lpk = a.head_dim * esz / 16;
     const bool single_ok = lpk >= 2 && pow2(lpk) && pow2(a.page_size) && a.max_blocks <= 4096;
     const bool decode = a.max_q_len == 1 && single_ok;
@@ -477,6 +481,8 @@ bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_
         int nsplit = 1, waves = 12;
         bool merge_kernel = false;
         decode_launch_shape(pairs, a.max_ctx_len, unmerged, &nsplit, &waves, &merge_kernel);
+        // (sigmoid weights have no sum to divide by afterwards: the kernel merges its own splits, however many)
+        if (a.shape != nullptr && a.shape->sigmoid) merge_kernel = false;
         unmerged = unmerged && nsplit > 1 && !merge_kernel;
         float* ws = decode_partials(nsplit > 1 ? static_cast<size_t>(pairs) * nsplit * (a.head_dim + 2) : 1, stream);
         int* counters = decode_counters(pairs, stream);

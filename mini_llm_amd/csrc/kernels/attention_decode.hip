@@ -64,7 +64,10 @@ __device__ __forceinline__ void merge_state(float& m, float& l, float (&o)[N], f
 
 // SHAPED: the scores are shaped before the softmax and a chunked mask may stand in for the window (score_shape.h);
 // the queries then come times the scale alone, and the shaped score goes to base 2 afterwards.
-template <typename T, int LPK, int UNR, bool SHAPED = false>
+// MODE 0: plain softmax; 1: shaped scores; 2: shaped scores whose weights are sigmoid(score + bias of the head), every
+// visible key on its own. The state keeps its form: the maximum stays 0 throughout, so every merge adds the outputs
+// as they are, the sum is unused and nothing is divided at the end.
+template <typename T, int LPK, int UNR, int MODE = 0>
 __global__ void __launch_bounds__(UNR > 8 ? 512 : DEC_MAX_WAVES * MLLM_WAVE)
 decode_attention_kernel(// the first 16 dwords arrive in registers with the wavefront: what the first loads need
                         const int* __restrict__ token_seq, const int* __restrict__ positions,
@@ -77,6 +80,7 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
                         T* __restrict__ k_pages_w, T* __restrict__ v_pages_w, int k_col, int v_col,
                         const int* __restrict__ slots, int partial_out, MllmScoreShape shape,
                         const float* __restrict__ gate, int ldg) {
+    constexpr bool SHAPED = MODE != 0, SIGMOID = MODE == 2;
     constexpr int EPL = Vec16<T>::N;        // elements per lane
     constexpr int DH = LPK * EPL;           // head size
     constexpr int KPW = MLLM_WAVE / LPK;    // keys per wavefront and load instruction
@@ -105,6 +109,7 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
     int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     if (SHAPED && shape.chunk > 0) lo = p - p % shape.chunk;
     const float r1 = (SHAPED && shape.r1) ? shape.r1[h] : 0.f, r2 = (SHAPED && shape.r1) ? shape.r2[h] : 0.f;
+    const float sbias = (SIGMOID && shape.score_bias) ? shape.score_bias[h] : 0.f;
     const int n_keys = p - lo + 1;
     const int per = (n_keys + nsplit - 1) / nsplit;
     const int kb = lo + split * per;
@@ -149,7 +154,8 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
     // Running state (maximum in base 2, sum, output slice). The maximum starts at a large
     // negative finite number, so that no difference of two of them is NaN.
     constexpr float NEG = -1.0e30f;
-    float m = NEG, l = 0.f, o[EPL];
+    constexpr float M0 = SIGMOID ? 0.f : NEG;       // an empty state's maximum
+    float m = M0, l = 0.f, o[EPL];
 #pragma unroll
     for (int e = 0; e < EPL; ++e) o[e] = 0.f;
 
@@ -180,18 +186,25 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
             d = group_sum<LPK>(d);
             const bool valid = j0 + u * group_keys + g < ke_pages;
             if (SHAPED) d = mllm_shaped_score<sizeof(T) == 2>(d, shape, r1, r2, valid ? p - (j0 + u * group_keys + g) : 0) * MLLM_LOG2E;
+            if (SIGMOID) {
+                const float w = 1.f / (1.f + exp2_for<T>(-(d + sbias * MLLM_LOG2E)));
+                dot[u] = valid ? w : 0.f;             // the weight itself
+                continue;
+            }
             dot[u] = valid ? d : NEG;
             mx = fmaxf(mx, dot[u]);
         }
         // one rescale of the state for the whole batch of keys
-        const float mn = fmaxf(m, mx);
-        const float a = exp2_for<T>(m - mn);
-        l *= a;
+        const float mn = SIGMOID ? 0.f : fmaxf(m, mx);
+        if (!SIGMOID) {
+            const float a = exp2_for<T>(m - mn);
+            l *= a;
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) o[e] *= a;
+            for (int e = 0; e < EPL; ++e) o[e] *= a;
+        }
 #pragma unroll
         for (int u = 0; u < UNR; ++u) {
-            const float pj = dot[u] > NEG ? exp2_for<T>(dot[u] - mn) : 0.f;
+            const float pj = SIGMOID ? dot[u] : dot[u] > NEG ? exp2_for<T>(dot[u] - mn) : 0.f;
             float vf[EPL];
             Vec16<T>::widen(vraw[u], vf);
             l += pj;
@@ -209,8 +222,9 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
         for (int e = 0; e < EPL; ++e) d = fmaf(qf[e], kf[e], d);
         d = group_sum<LPK>(d);
         if (SHAPED) d = mllm_shaped_score<sizeof(T) == 2>(d, shape, r1, r2, 0) * MLLM_LOG2E;
-        const float mn = fmaxf(m, d);
-        const float a = exp2_for<T>(m - mn), pj = exp2_for<T>(d - mn);
+        const float mn = SIGMOID ? 0.f : fmaxf(m, d);
+        const float a = SIGMOID ? 1.f : exp2_for<T>(m - mn);
+        const float pj = SIGMOID ? 1.f / (1.f + exp2_for<T>(-(d + sbias * MLLM_LOG2E))) : exp2_for<T>(d - mn);
         l = l * a + pj;
 #pragma unroll
         for (int e = 0; e < EPL; ++e) o[e] = o[e] * a + pj * vf[e];
@@ -237,7 +251,7 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
         if (wave == 0) {
             // lane group G takes the state of wavefront G, G + KPW, ... (all reads at once), then
             // the groups are merged as above
-            m = NEG; l = 0.f;
+            m = M0; l = 0.f;
 #pragma unroll
             for (int e = 0; e < EPL; ++e) o[e] = 0.f;
             for (int w = g; w < n_waves; w += KPW) {
@@ -270,11 +284,11 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
     }
     if (nsplit == 1) {
         if (wave == 0 && g == 0) {
-            const float inv = 1.0f / l;
+            const float inv = SIGMOID ? 1.f : 1.0f / l;
 #pragma unroll
             for (int e = 0; e < EPL; ++e) {
                 float r = o[e] * inv;
-                if (SHAPED && gate != nullptr) r *= 1.f / (1.f + __expf(-gate[static_cast<size_t>(t) * ldg + h * DH + c * EPL + e]));
+                if (SHAPED && gate != nullptr) r *= 1.f / (1.f + __expf(-gate[static_cast<size_t>(t) * ldg + (shape.gate_per_head ? h : h * DH + c * EPL + e)]));
                 op[e] = from_float<T>(r);
             }
         }
@@ -301,7 +315,7 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
     if (!sm_last) return;
     // Last workgroup of this (token, head): lane group G takes split G (all loads in flight at
     // once), then the same merge as above.
-    m = NEG; l = 0.f;
+    m = M0; l = 0.f;
 #pragma unroll
     for (int e = 0; e < EPL; ++e) o[e] = 0.f;
     for (int s0 = 0; s0 < nsplit; s0 += n_waves * KPW) {
@@ -319,11 +333,11 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
     }
     block_merge();
     if (wave == 0 && g == 0) {
-        const float inv = 1.0f / l;
+        const float inv = SIGMOID ? 1.f : 1.0f / l;
 #pragma unroll
         for (int e = 0; e < EPL; ++e) {
             float r = o[e] * inv;
-            if (SHAPED && gate != nullptr) r *= 1.f / (1.f + __expf(-gate[static_cast<size_t>(t) * ldg + h * DH + c * EPL + e]));
+            if (SHAPED && gate != nullptr) r *= 1.f / (1.f + __expf(-gate[static_cast<size_t>(t) * ldg + (shape.gate_per_head ? h : h * DH + c * EPL + e)]));
             op[e] = from_float<T>(r);
         }
     }
@@ -344,8 +358,9 @@ static int launch_decode(int lpk, dim3 grid, int waves, hipStream_t stream, cons
             ws_o, ws_ml, counters, k_pages_w, v_pages_w, k_col, v_col, slots, partial_out, sh, gate, ldg
 #define DEC_CASE(L)                                                                                    \
     case L:                                                                                            \
-        if (shape) decode_attention_kernel<T, L, 8, true><<<grid, waves * MLLM_WAVE, 0, stream>>>(DEC_ARGS); \
-        else decode_attention_kernel<T, L, 8, false><<<grid, waves * MLLM_WAVE, 0, stream>>>(DEC_ARGS);  \
+        if (shape && shape->sigmoid) decode_attention_kernel<T, L, 8, 2><<<grid, waves * MLLM_WAVE, 0, stream>>>(DEC_ARGS); \
+        else if (shape) decode_attention_kernel<T, L, 8, 1><<<grid, waves * MLLM_WAVE, 0, stream>>>(DEC_ARGS); \
+        else decode_attention_kernel<T, L, 8, 0><<<grid, waves * MLLM_WAVE, 0, stream>>>(DEC_ARGS);      \
         return 0;
     switch (lpk) {
         DEC_CASE(2) DEC_CASE(4) DEC_CASE(8) DEC_CASE(16) DEC_CASE(32) DEC_CASE(64)
@@ -434,6 +449,8 @@ int mllm_decode_attention(const void* q, int q_stride, int q_col, const void* k_
     if (shape && window > 0 && shape->chunk > 0) return -1;
     // (a gate goes with shaped scores, and with a result that this kernel finishes itself)
     if (gate != nullptr && (shape == nullptr || partial_out)) return -1;
+    // (weights that are not normalised leave no sum for another kernel to divide by)
+    if (shape && shape->sigmoid && partial_out) return -1;
     int rc;
     if (dtype == MLLM_F32)
         rc = launch_decode<float>(lpk, grid, waves, stream, (const float*)q, q_stride, q_col, (const float*)k_pages,

@@ -42,7 +42,10 @@ union Frag8 {
 // prefetched tiles in registers instead of private memory.)
 // SHAPED: the scores are shaped before the softmax (score_shape.h: cap, distance bias), a chunked mask may stand in
 // for the window, and the result may be multiplied by the sigmoid of a gate (fp32 rows, one value per output column).
-template <int DH, int NW, bool SHAPED = false>
+// MODE 0: plain softmax; 1: shaped scores; 2: shaped scores whose weights are sigmoid(score + bias of the head), every
+// visible key on its own: no running maximum, no sum, nothing to rescale, and the states of two wavefronts simply add.
+// The weights are fp32 until they are packed for the second product, as the softmax's are.
+template <int DH, int NW, int MODE = 0>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, (DH >= 128 && NW == 4) ? 1 : 2)))
 prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
                          const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages, int kv_dim,
@@ -51,6 +54,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
                          int n_heads, int n_kv_heads, int page_size, float scale_log2e, int window,
                          bf16_t* __restrict__ out, int out_stride, MllmScoreShape shape, float scale,
                          const float* __restrict__ gate, int ldg) {
+    constexpr bool SHAPED = MODE != 0, SIGMOID = MODE == 2;
     constexpr int KS = DH / 32;            // k steps of S^T
     constexpr int DT = DH / 16;            // 16-dim tiles of O^T
     constexpr int KSTRIDE = DH + 8;
@@ -93,6 +97,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
     const int chunk = SHAPED ? shape.chunk : 0;
     if (chunk > 0) k_lo = p_first - p_first % chunk;
     const float r1 = (SHAPED && shape.r1) ? shape.r1[blockIdx.x] : 0.f, r2 = (SHAPED && shape.r1) ? shape.r2[blockIdx.x] : 0.f;
+    const float sbias = (SIGMOID && shape.score_bias) ? shape.score_bias[blockIdx.x] : 0.f;
     // (shaped scores are in base 2 already when they meet the exponent)
     const float sl = SHAPED ? 1.f : scale_log2e;
     // The sequence's block table goes to LDS first: the gathers below then depend on an LDS read,
@@ -191,6 +196,16 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
             for (int r = 0; r < 4; ++r) {
                 s[nt][r] = acc[r];                   // raw dot product; the scale is applied with the exponent
                 const int j = j_base + 16 * (nt0 + nt) + 4 * G + r;
+                if constexpr (SIGMOID) {
+                    const float z = mllm_shaped_score<true>(acc[r] * scale, shape, r1, r2, max(p - j, 0)) + sbias;
+                    float w = __builtin_amdgcn_rcpf(1.f + fast_exp2(-z * MLLM_LOG2E));
+                    if (MASKED) {
+                        const bool seen = q_ok && j <= p && (window <= 0 || j > p - window) && (chunk <= 0 || j >= p - p % chunk);
+                        if (!seen) w = 0.f;
+                    }
+                    s[nt][r] = w;
+                    continue;
+                }
                 if (SHAPED) s[nt][r] = mllm_shaped_score<true>(acc[r] * scale, shape, r1, r2, max(p - j, 0)) * MLLM_LOG2E;
                 if (MASKED) {
                     const bool seen = q_ok && j <= p && (window <= 0 || j > p - window) && (chunk <= 0 || j >= p - p % chunk);
@@ -199,6 +214,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
                 tile_max = fmaxf(tile_max, s[nt][r]);
             }
         }
+        if constexpr (!SIGMOID) {
         // the four lane groups of a query agree on the maximum
         tile_max = rows_max(tile_max);
         const float m_new = fmaxf(m, tile_max * sl);        // the scale is positive
@@ -218,6 +234,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
+        }
 
         // O^T += V^T P^T over slabs of 32 keys. k slot i of lane group G stands for key
         // 32*slab + 4*G + i (i < 4) or 32*slab + 16 + 4*G + i - 4 (i >= 4) in both operands.
@@ -308,7 +325,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
         const float m1 = state[0];
         const float m_new = fmaxf(m, m1);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float a0 = fast_exp2(m - m_use), a1 = fast_exp2(m1 - m_use);
+        const float a0 = SIGMOID ? 1.f : fast_exp2(m - m_use), a1 = SIGMOID ? 1.f : fast_exp2(m1 - m_use);
         l = l * a0 + state[1] * a1;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
@@ -317,13 +334,17 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
     }
     l = rows_sum(l);
     if (!q_ok) return;
-    const float inv = 1.0f / l;
+    const float inv = SIGMOID ? 1.f : 1.0f / l;
+    const bool head_gate = SHAPED && gate != nullptr && shape.gate_per_head;
+    const float hg = head_gate ? 1.f / (1.f + __expf(-gate[static_cast<size_t>(q_begin + qi) * ldg + blockIdx.x])) : 1.f;
     // o[dt][r] is dimension 16*dt + 4*G + r of this lane's query
     bf16_t* orow = out + static_cast<size_t>(q_begin + qi) * out_stride + h * DH;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
         float g4[4] = {1.f, 1.f, 1.f, 1.f};
-        if (SHAPED && gate != nullptr) {
+        if (head_gate) {
+            g4[0] = g4[1] = g4[2] = g4[3] = hg;
+        } else if (SHAPED && gate != nullptr) {
             const float4 gv = *reinterpret_cast<const float4*>(gate + static_cast<size_t>(q_begin + qi) * ldg + blockIdx.x * DH + 16 * dt + 4 * G);
             g4[0] = 1.f / (1.f + __expf(-gv.x)); g4[1] = 1.f / (1.f + __expf(-gv.y));
             g4[2] = 1.f / (1.f + __expf(-gv.z)); g4[3] = 1.f / (1.f + __expf(-gv.w));
@@ -350,7 +371,7 @@ int mllm_prefill_attention_bf16(const void* q, int q_stride, int q_col, const vo
     if (n_seqs <= 0 || n_tiles_upper <= 0) return 0;
     // (the gate is read 16 bytes at a time)
     if (shape == nullptr && gate != nullptr) return -1;
-    if (gate != nullptr && (ldg % 4 != 0 || (reinterpret_cast<uintptr_t>(gate) & 15) != 0)) return -1;
+    if (gate != nullptr && !shape->gate_per_head && (ldg % 4 != 0 || (reinterpret_cast<uintptr_t>(gate) & 15) != 0)) return -1;
     if (shape && window > 0 && shape->chunk > 0) return -1;
     const MllmScoreShape sh = shape ? *shape : MllmScoreShape{0.f, 0, nullptr, nullptr};
     if (n_heads % n_kv_heads != 0 || n_tiles_upper > 65535) return -1;
@@ -375,7 +396,9 @@ int mllm_prefill_attention_bf16(const void* q, int q_stride, int q_col, const vo
     } while (0)
 #define PF_CASE(D, W, KEY)                                                                                  \
     case KEY: {                                                                                             \
-        if (shape) PF_LAUNCH(D, W, true); else PF_LAUNCH(D, W, false);                                      \
+        if (shape && shape->sigmoid) PF_LAUNCH(D, W, 2);                                                    \
+        else if (shape) PF_LAUNCH(D, W, 1);                                                                 \
+        else PF_LAUNCH(D, W, 0);                                                                            \
         break;                                                                                              \
     }
     // Eight wavefronts (two per 16 queries, half a key tile each) shorten the longest workgroup's chain of

@@ -50,7 +50,7 @@ class AttentionArgsC(ctypes.Structure):
 
 
 class ScoreShapeC(ctypes.Structure):
-    _fields_ = [("softcap", _f), ("chunk", _i), ("r1", _vp), ("r2", _vp)]
+    _fields_ = [("softcap", _f), ("chunk", _i), ("r1", _vp), ("r2", _vp), ("sigmoid", _i), ("score_bias", _vp), ("gate_per_head", _i)]
 
 
 _lib = None
@@ -459,10 +459,18 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
                 if t_.dtype != torch.float32 or t_.numel() != n_heads or not t_.is_contiguous():
                     raise KernelError(f"{n_} must be contiguous float32 [n_heads]")
             sh.r1, sh.r2 = r1.data_ptr(), r2.data_ptr()
+        sh.sigmoid, sh.gate_per_head = (1 if shape.get("sigmoid") else 0), (1 if shape.get("gate_per_head") else 0)
+        sb = shape.get("score_bias")
+        if sb is not None:
+            _gpu(sb)
+            if sb.dtype != torch.float32 or sb.numel() != n_heads or not sb.is_contiguous():
+                raise KernelError("score_bias must be contiguous float32 [n_heads]")
+            sh.score_bias = sb.data_ptr()
         a.shape = ctypes.addressof(sh)
     if gate is not None:
         _gpu(gate)
-        if gate.dtype != torch.float32 or gate.dim() != 2 or gate.shape[0] != T or gate.shape[1] < n_heads * head_dim or gate.stride(1) != 1:
+        per_head = shape is not None and shape.get("gate_per_head")
+        if gate.dtype != torch.float32 or gate.dim() != 2 or gate.shape[0] != T or gate.shape[1] < (n_heads if per_head else n_heads * head_dim) or gate.stride(1) != 1:
             raise KernelError("gate must be float32 [T, >= n_heads*head_dim]")
         a.gate, a.gate_stride = gate.data_ptr(), gate.stride(0)
     push_tuning()

@@ -113,9 +113,16 @@ def paged_attention(q, q_col, n_heads, n_kv_heads, head_dim, k_pages, v_pages, p
                 s = shape["softcap"] * torch.tanh(s / shape["softcap"])
             if shape and shape.get("r1") is not None:
                 s = s - shape["r1"][h].to(PRECISE) * torch.log1p(shape["r2"][h].to(PRECISE) * (p - js).to(PRECISE))
-            w = torch.softmax(s, dim=0)
+            if shape and shape.get("sigmoid"):
+                # every visible key on its own: sigmoid(score + the head's bias), not normalised over the keys
+                bias = shape["score_bias"][h].to(PRECISE) if shape.get("score_bias") is not None else 0.0
+                w = torch.sigmoid(s + bias)
+            else:
+                w = torch.softmax(s, dim=0)
             o = w @ v
-            if gate is not None:
+            if gate is not None and shape and shape.get("gate_per_head"):
+                o = o * torch.sigmoid(gate[t, h].to(PRECISE))
+            elif gate is not None:
                 o = o * torch.sigmoid(gate[t, h * head_dim:(h + 1) * head_dim].to(PRECISE))
             out[t, h * head_dim:(h + 1) * head_dim] = o.to(out.dtype)
     return out

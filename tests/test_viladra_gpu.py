@@ -101,6 +101,30 @@ def test_window_and_page_borders_with_peaked_scores(dirs, page):
                                tol=vc.TOL_PEAKED)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["PEAKED_TILES_32", "PEAKED_TILES_64", "PEAKED_TILES_128"])
+def test_window_borders_at_the_tiled_kernels_head_sizes(dirs, name, dtype):
+    """Small windows with peaked scores at head sizes 32, 64 and 128, where bfloat16 prompts run on tiles of 64
+    queries by 128 keys and single tokens on split keys: prompts of 300 tokens (windows that straddle a key tile's
+    and a page's border), portions of many sizes, decoding, and a mixed batch. The plain model with the window one
+    key wider fails the same comparison by far."""
+    cfg, d = getattr(vc, name), dirs(name)
+    reqs = vc.requests(cfg["vocab"], [300, 130, 64, 7], seed=25)
+    mixed, _ = ru.trace_mixed(reqs, seed=8, max_live=4, tail=6)
+    for label, steps in (("whole", ru.trace_whole(reqs)), ("decode", ru.trace_decode_tail(reqs, tail=30)),
+                         ("chunks", ru.trace_chunks(reqs, seed=5, sizes=(2, 70, 3, 129, 16, 64))), ("mixed", mixed)):
+        runner = _runner(d, dtype, n_pages=-(-ru.peak_tokens(steps) // 16) + 4, page=16)
+        vc.check_against_plain(d, reqs, steps, ru.run_in_process(runner, steps), dtype, cfg["vocab"], f"{name} {label}")
+    if dtype == "bfloat16":
+        c, w = pv.read_model(d)
+        wider = copy.deepcopy(c)
+        wider["layers"][0]["mixer"]["mask"]["size"] += 1
+        toks = reqs["r0"]
+        a, b = pv.forward(c, w, toks).numpy(), pv.forward(wider, w, toks).numpy()
+        errs = np.array([vc.row_error(b[p], a[p]) for p in range(10, len(toks))])
+        assert (errs > 3 * vc.TOL["bfloat16"]).mean() > 0.25, errs
+
+
 @pytest.mark.parametrize("page", [4, 16])
 def test_far_keys_among_hundreds(dirs, page):
     """A window of 300 keys with peaked scores, a recurrence that never forgets and ones that forget slowly: a key

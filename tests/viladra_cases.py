@@ -69,6 +69,12 @@ MIXED_B = model([
 # peaking; the score bias lies around -2, so most other keys weigh little): a window that is one key off, or a key lost
 # at a page's border, changes a row
 PEAKED = model([attention(window=5, scale=3.0), attention(window=16, scale=3.0, heads=2, kv_heads=1, vdim=16)], width=32)
+# the same at the head sizes that the matrix-core tiles and the split-key kernel take in bfloat16 (32, 64, 128; keys
+# and values of one width), one layer each so that a row shows its own window: one key more or less in a window
+# changes a third to two thirds of the rows by more than three times the bfloat16 tolerance
+PEAKED_TILES_32 = model([attention(window=9, scale=0.8, heads=4, kv_heads=2, dim=32, vdim=32)], width=64)
+PEAKED_TILES_64 = model([attention(window=5, scale=0.6, heads=2, kv_heads=1, dim=64, vdim=64)], width=64)
+PEAKED_TILES_128 = model([attention(window=3, scale=0.4, heads=2, kv_heads=2, dim=128, vdim=128)], width=32)
 # the same with a window of hundreds of keys, and recurrences that forget slowly: a token far back carries a row
 PEAKED_FAR = model([attention(window=300, scale=3.0), retention(heads=2, dim=8, vdim=8, decay=[0.998046875, 1.0]),
                     gla(heads=2, dim=8, vdim=8, tau=64.0)], width=32)
