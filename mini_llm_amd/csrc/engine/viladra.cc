@@ -245,6 +245,7 @@ void viladra_assemble(const Json& config, const std::map<std::string, Tensor2>& 
         p.tensor["weight"] = t.at(name);
         return build_norm("rmsnorm", p);
     };
+    Tensor2 no_conv;
     Params mix;
     mix.num["passes"] = static_cast<double>(c.layers.size());
     for (size_t i = 0; i < c.layers.size(); ++i) {
@@ -314,6 +315,11 @@ void viladra_assemble(const Json& config, const std::map<std::string, Tensor2>& 
         if (c.taps > 0) {
             b.tensor["mixer_conv"] = t.at(L + "canon1");
             if (l.mlp.present) b.tensor["ff_conv"] = t.at(L + "canon2");
+        } else if (dtype != F32) {
+            // (no input convolution: one tap of weight zero hands the stream on in the compute dtype)
+            if (no_conv.data == nullptr) { const Tensor2 z = out.store.zeros(D); no_conv = Tensor2(z.data, F32, D, 1); }
+            b.tensor["mixer_conv"] = no_conv;
+            if (l.mlp.present) b.tensor["ff_conv"] = no_conv;
         }
         m.layers.push_back(build_block("post_norm", std::move(mixer), std::move(ff), std::move(norms), b));
         mix.tensor["w" + std::to_string(i)] = t.at(L + "dwa");

@@ -68,9 +68,9 @@ def test_written_folder_checks_a_missing_tensor_is_named_and_the_rank_is_the_che
     assert arch == "Viladra" and n_tensors == len(describe_config(vc.MIXED_B)["tensors"])
     from safetensors.torch import load_file, save_file
     t = load_file(str(tmp_path / "m" / "model.safetensors"))
-    del t["l1.mlp.e7.down"]
+    del t["l1.mlp.e6.down"]
     save_file(t, str(tmp_path / "m" / "model.safetensors"))
-    with pytest.raises(WeightsError, match="l1.mlp.e7.down"):
+    with pytest.raises(WeightsError, match="l1.mlp.e6.down"):
         check_model_dir(d)
     # a low-rank map of another rank than the configuration would write is taken as stored; a height that is wrong is not
     d2 = write_random_model(dict(vc.ONLY_GLA), str(tmp_path / "g"), 1)

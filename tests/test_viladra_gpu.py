@@ -45,7 +45,7 @@ def _families(reqs, seed):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["ONLY_RETENTION", "ONLY_RETENTION_PLAIN", "ONLY_GLA", "ONLY_GLA_WIDE", "ONLY_ATTENTION",
-                                  "ONLY_ATTENTION_SQUARE", "ONLY_EXPERTS", "ONLY_EXPERTS_ALL", "ONE_EXPERT"])
+                                  "ONLY_ATTENTION_SQUARE", "ONLY_EXPERTS", "ONLY_EXPERTS_ALL", "ONE_EXPERT", "NO_CONVOLUTION"])
 def test_each_mechanism_alone(dirs, name, dtype):
     cfg, d = getattr(vc, name), dirs(name)
     reqs = vc.requests(cfg["vocab"], [1, 2, 3, 9, 37, 64, 65, 150], seed=5)

@@ -36,7 +36,9 @@ def moe(experts=4, top=2, ff=24, shared=40, scale=1.5):
 
 def model(layers, vocab=300, width=64, eps=1e-5, taps=4, embed_scale=0.7, softcap=20.0):
     c = {"architecture": "Viladra", "vocab": vocab, "width": width, "norm": {"eps": eps}, "layers": layers,
-         "embedding": {"scale": embed_scale}, "canon": {"taps": taps}}
+         "embedding": {"scale": embed_scale}}
+    if taps is not None:
+        c["canon"] = {"taps": taps}
     if softcap is not None:
         c["logit_softcap"] = softcap
     return c
@@ -51,6 +53,7 @@ ONLY_ATTENTION = model([attention()])
 ONLY_ATTENTION_SQUARE = model([attention(heads=3, kv_heads=3, dim=24, vdim=24, window=40)], width=48, taps=1, embed_scale=1.0)
 ONLY_EXPERTS = model([retention(mlp=moe())])
 ONLY_EXPERTS_ALL = model([gla(mlp=moe(experts=3, top=3, ff=16, shared=None, scale=1.0))], width=32)      # every expert chosen, no shared one
+NO_CONVOLUTION = model([gla(mlp=moe(experts=3, top=1, ff=16, shared=8)), attention(window=7)], width=32, taps=None)
 ONE_EXPERT = model([attention(mlp=moe(experts=1, top=1, ff=32, shared=16, scale=3.0))], width=32)
 # several layers in orders of their own: what a layer hands on is a weighted sum over everything before it
 MIXED_A = model([
@@ -62,7 +65,7 @@ MIXED_A = model([
 ], vocab=257, width=64, eps=1e-6, taps=3)
 MIXED_B = model([
     attention(heads=1, kv_heads=1, dim=48, vdim=16, window=33),
-    retention(heads=1, dim=64, vdim=24, decay=[0.99], base=500.0, dims=64, mlp=moe(experts=8, top=3, ff=16, shared=32, scale=2.5)),
+    retention(heads=1, dim=64, vdim=24, decay=[0.99], base=500.0, dims=64, mlp=moe(experts=7, top=3, ff=16, shared=32, scale=1.75)),
     retention(heads=5, dim=16, vdim=8, dims=16, mlp=moe(experts=3, top=2, ff=24)),
 ], vocab=513, width=48, taps=2, embed_scale=0.25, softcap=5.0)
 # scores that single keys dominate (queries and keys are normed, so |q.k| is about dim at most: the scale does the
@@ -88,8 +91,8 @@ ODD = model([
 ], vocab=101, width=43, taps=6)
 # the sizes of a larger model's layers: heads of 64 and 128, pages of many sizes
 LARGER = model([
-    gla(heads=4, dim=64, vdim=128, tau=16.0, rank=16, mlp=moe(experts=8, top=2, ff=64, shared=128)),
-    attention(heads=4, kv_heads=2, dim=64, vdim=64, window=100, mlp=moe(experts=8, top=2, ff=64, shared=128)),
+    gla(heads=4, dim=64, vdim=128, tau=12.0, rank=16, mlp=moe(experts=6, top=2, ff=96, shared=160)),
+    attention(heads=4, kv_heads=2, dim=64, vdim=64, window=100, mlp=moe(experts=6, top=2, ff=96, shared=160)),
     retention(heads=2, dim=128, vdim=128, dims=64, decay=[0.96875, 0.998046875]),
     attention(heads=2, kv_heads=1, dim=128, vdim=128, window=150),
 ], vocab=211, width=256)
