@@ -91,6 +91,9 @@ int mllm_conv_residual(const float* in, int ld, int C, const float* w, int taps,
 int mllm_rmsnorm_conv_single(const float* x, int ldx, const float* wn, float eps, int C, const float* wc, int taps,
                              const int* state_slots, float* state, size_t slot_floats, void* out, int ldo, int out_dtype, int T,
                              int write, hipStream_t stream);
+int mllm_stream_conv_single(float* x, int ldx, const float* y, int ldy, const float* wn, float eps, int C, const float* wc, int taps,
+                            const int* state_slots, float* state, size_t slot_floats, void* out, int ldo, int out_dtype, int T,
+                            int write, hipStream_t stream);
 int mllm_ssm_scan(const float* xbc, int ldx, const float* raw_dt, int ldd, const float* dt_bias, const float* A_log,
                   const float* Dskip, const int* cu_q, const int* state_slots, float* state, size_t slot_floats,
                   size_t scan_offset, float* y, int ldy, size_t part_stride, int T, int B, int max_q_len, int H, int P, int N,

@@ -254,6 +254,11 @@ void conv_residual(const Tensor2& in, const Tensor2& weight, const StateArgs& st
 // False (and nothing done): sizes the kernel is not made for (more than 8 taps, rows wider than 2,048).
 bool rmsnorm_conv_single(const Tensor2& x, const float* norm_weight, float eps, const Tensor2& weight, const StateArgs& st,
                          const Tensor2& out, hipStream_t stream);
+// For the same kind of step, a convolution that reads the stream itself: out = x + conv(x); and, with `y` (a sub-layer's
+// result, fp32, x's shape) and a norm's weight, behind x += y / sqrt(mean(y^2) + eps) * norm_weight (x is written) in
+// the same kernel. False (and nothing done): sizes the kernel is not made for, as above.
+bool stream_conv_single(const Tensor2& x, const Tensor2* y, const float* norm_weight, float eps, const Tensor2& weight,
+                        const StateArgs& st, const Tensor2& out, hipStream_t stream);
 // x += mult * sum_k rmsnorm(y_k) * w_k: n inputs of x's shape one behind the other in `ys` ([n * rows, size] fp32), their
 // weights one behind the other in `weights` ([n * size]); 2 to 4 inputs, rows of up to 2,048 columns.
 void rmsnorm_add_many(const Tensor2& ys, const float* weights, int n, float mult, float eps, const Tensor2& x, hipStream_t stream);

@@ -71,6 +71,30 @@ bool rmsnorm_conv_single(const Tensor2& x, const float* norm_weight, float eps, 
     return true;
 }
 
+bool stream_conv_single(const Tensor2& x, const Tensor2* y, const float* norm_weight, float eps, const Tensor2& weight,
+                        const StateArgs& st, const Tensor2& out, hipStream_t stream) {
+    need_f32(x, "stream_conv_single: the stream");
+    need_f32(weight, "stream_conv_single: the taps");
+    need_act(out, "stream_conv_single: out");
+    const int C = i32(weight.rows), taps = i32(weight.cols);
+    if (!weight.contiguous() || taps < 1 || taps > 16) fail("stream_conv_single: taps [channels, 1 to 16] contiguous are needed");
+    if (x.cols != C || out.cols != C || out.rows != x.rows) fail("stream_conv_single: stream and out must be [T, %d]", C);
+    if (y != nullptr) {
+        need_f32(*y, "stream_conv_single: the sub-layer's result");
+        if (y->rows != x.rows || y->cols != C || norm_weight == nullptr) fail("stream_conv_single: the result must be [T, %d] and comes with a norm's weight", C);
+    }
+    if (x.rows != st.n_seqs || st.state_slots == nullptr) fail("stream_conv_single: every sequence of the step must bring one token");
+    if (taps > 1 && (st.state == nullptr || st.slot_floats < static_cast<size_t>(taps - 1) * C))
+        fail("stream_conv_single: a state slot holds %zu floats, %zu are needed", st.slot_floats, static_cast<size_t>(taps - 1) * C);
+    const int rc = mllm_stream_conv_single(static_cast<float*>(x.data), i32(x.stride), y ? static_cast<const float*>(y->data) : nullptr,
+                                           y ? i32(y->stride) : 0, y ? norm_weight : nullptr, eps, C, static_cast<const float*>(weight.data), taps,
+                                           st.state_slots, st.state, st.slot_floats, out.data, i32(out.stride), out.dtype, i32(x.rows),
+                                           st.write ? 1 : 0, stream);
+    if (rc == -2) return false;
+    check(rc, "stream_conv_single");
+    return true;
+}
+
 void rmsnorm_add_many(const Tensor2& ys, const float* weights, int n, float mult, float eps, const Tensor2& x, hipStream_t stream) {
     need_f32(ys, "rmsnorm_add_many: the inputs");
     need_f32(x, "rmsnorm_add_many: x");

@@ -212,6 +212,13 @@ public:
         (void)x; (void)taps; (void)st; (void)out; (void)s;
         return false;
     }
+    // For the same kind of step and a norm BEHIND a sub-layer: x += norm(y) (y: the sub-layer's result, fp32) and
+    // out = x + conv(x), the next sub-layer's input, in one kernel. False: no such kernel, nothing was done.
+    virtual bool add_conv_single(const Tensor2& y, const Tensor2& x, const Tensor2& taps, const StateArgs& st, const Tensor2& out,
+                                 hipStream_t s) const {
+        (void)y; (void)x; (void)taps; (void)st; (void)out; (void)s;
+        return false;
+    }
     // out = epilogue(lin(norm(x[rows]))); a norm with a fused kernel overrides this
     // (kv: a key/value scatter of the linear map, passed through to it)
     virtual void linear(const Tensor2& x, const Linear& lin, const Tensor2& out, int epilogue, const int* rows,

@@ -38,6 +38,11 @@ public:
         if (x.cols != size_) fail("rmsnorm: rows of %lld, the norm is %d wide", (long long)x.cols, size_);
         return rmsnorm_conv_single(x, weight_, eps_, taps, st, out, s);
     }
+    bool add_conv_single(const Tensor2& y, const Tensor2& x, const Tensor2& taps, const StateArgs& st, const Tensor2& out,
+                         hipStream_t s) const override {
+        if (y.cols != size_) fail("rmsnorm: rows of %lld, the norm is %d wide", (long long)y.cols, size_);
+        return stream_conv_single(x, &y, weight_, eps_, taps, st, out, s);
+    }
     void linear(const Tensor2& x, const Linear& lin, const Tensor2& out, int epilogue, const int* rows,
                 const KvScatter* kv, Arena& arena, hipStream_t s) const override {
         if (kv != nullptr) { Norm::linear(x, lin, out, epilogue, rows, kv, arena, s); return; }
@@ -185,11 +190,20 @@ public:
             mixer_->forward_set(h, step, rest, y, write, arena, s);
         }
         arena.release(mark);
-        norm1_->add_scaled(y, nullptr, 1.f, x, false, s);
+        // every sequence brings one token: the norm behind the mixer and the feed-forward's convolution in one kernel
+        Tensor2 fused;
+        if (ff_ && conv2_.data != nullptr && single_tokens(step)) {
+            fused = arena.tensor(dtype_, x.rows, x.cols);
+            if (!norm1_->add_conv_single(y, x, conv2_, state_args(conv1_bytes_, step, cache, write), fused, s)) {
+                fused = Tensor2();
+                arena.release(mark);
+            }
+        }
+        if (fused.data == nullptr) norm1_->add_scaled(y, nullptr, 1.f, x, false, s);
         StageTimes::get().mark("post_norm", s);
         if (ff_) {
             {
-                NormedInput h(input(x, conv2_, conv1_bytes_, step, cache, write, arena, s));
+                NormedInput h(fused.data != nullptr ? fused : input(x, conv2_, conv1_bytes_, step, cache, write, arena, s));
                 ff_->forward_set(h, step, y, arena, s);
             }
             arena.release(mark);
@@ -236,13 +250,20 @@ private:
         }
         if (x.cols != conv.rows) fail("the input convolution has %lld channels, the stream %lld", (long long)conv.rows, (long long)x.cols);
         Tensor2 hc = arena.tensor(dtype_, x.rows, x.cols);
+        const StateArgs st = state_args(state_at, step, cache, write);
+        // (single tokens: a kernel that asks for all its loads at once)
+        if (!(single_tokens(step) && stream_conv_single(x, nullptr, nullptr, 0.f, conv, st, hc, s))) conv_residual(x, conv, st, hc, s);
+        StageTimes::get().mark("input_conv", s);
+        return hc;
+    }
+    static bool single_tokens(const StepView& step) { return step.max_q_len == 1 && step.n_tokens == step.n_seqs; }
+    // The step's arrays and the carried rows that lie `state_at` bytes into the layer's slot.
+    static StateArgs state_args(size_t state_at, const StepView& step, const CacheView& cache, bool write) {
         StateArgs st;
         st.token_seq = step.token_seq; st.cu_q = step.cu_q; st.state_slots = step.state_slots; st.n_seqs = step.n_seqs;
         st.max_q_len = step.max_q_len; st.state = reinterpret_cast<float*>(static_cast<char*>(cache.state) + state_at);
         st.slot_floats = cache.slot_bytes / 4; st.n_slots = cache.n_slots; st.write = write;
-        conv_residual(x, conv, st, hc, s);
-        StageTimes::get().mark("input_conv", s);
-        return hc;
+        return st;
     }
     std::unique_ptr<Mixer> mixer_;
     std::unique_ptr<FeedForward> ff_;

@@ -74,9 +74,12 @@ __global__ void conv_residual_kernel(const float* __restrict__ in, int ld, int C
 // block are issued together, without conditions, from clamped (always valid) places, and masked where they are used
 // (a load under a condition, or in a loop of unknown length, is waited for before the next is asked for); TAPS is a
 // constant for that reason.
-template <typename OutT, int WAVES, int TAPS, int NB>
+// MODE 0: as above. MODE 1, a norm BEHIND a sub-layer and the next sub-layer's convolution: the stream's row becomes
+// x + y / sqrt(mean(y^2) + eps) * wn (y: the sub-layer's result; x is written back), and h is that row. MODE 2: no norm,
+// h = x.
+template <typename OutT, int WAVES, int TAPS, int NB, int MODE>
 __global__ void __launch_bounds__(64 * WAVES)
-rmsnorm_conv_single_kernel(const float* __restrict__ x, int ldx, const float* __restrict__ wn, float eps, int C,
+rmsnorm_conv_single_kernel(float* x, int ldx, const float* __restrict__ y, int ldy, const float* __restrict__ wn, float eps, int C,
                            const float* __restrict__ wc, const int* __restrict__ state_slots, float* __restrict__ state,
                            size_t slot_floats, OutT* __restrict__ out, int ldo, int T, int write) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MLLM_WAVE), lane = threadIdx.x % MLLM_WAVE;
@@ -84,18 +87,31 @@ rmsnorm_conv_single_kernel(const float* __restrict__ x, int ldx, const float* __
     if (t >= T) return;
     const int slot = state_slots[t];
     if (slot < 0) return;
-    const float* xr = x + static_cast<size_t>(t) * ldx;
-    float xv[NB][8];
+    float* xr = x + static_cast<size_t>(t) * ldx;
+    float xv[NB][8], yv[MODE == 1 ? NB : 1][8];
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
         for (int u = 0; u < 8; ++u) xv[b][u] = xr[min(512 * b + lane + 64 * u, C - 1)];
-    float ss = 0.f;
+    if (MODE == 1) {
+        const float* yr = y + static_cast<size_t>(t) * ldy;
 #pragma unroll
-    for (int b = 0; b < NB; ++b)
+        for (int b = 0; b < NB; ++b)
 #pragma unroll
-        for (int u = 0; u < 8; ++u) ss += (512 * b + lane + 64 * u < C) ? xv[b][u] * xv[b][u] : 0.f;
-    const float inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(C) + eps);
+            for (int u = 0; u < 8; ++u) yv[b][u] = yr[min(512 * b + lane + 64 * u, C - 1)];
+    }
+    float inv = 1.f;
+    if (MODE != 2) {
+        float ss = 0.f;
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const float z = MODE == 1 ? yv[b][u] : xv[b][u];
+                ss += (512 * b + lane + 64 * u < C) ? z * z : 0.f;
+            }
+        inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(C) + eps);
+    }
     float* carried = state + static_cast<size_t>(slot) * slot_floats;
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
@@ -105,7 +121,7 @@ rmsnorm_conv_single_kernel(const float* __restrict__ x, int ldx, const float* __
 #pragma unroll
         for (int u = 0; u < 8; ++u) idx[u] = min(512 * b + lane + 64 * u, C - 1);
 #pragma unroll
-        for (int u = 0; u < 8; ++u) g[u] = wn[idx[u]];
+        for (int u = 0; u < 8; ++u) g[u] = MODE == 2 ? 1.f : wn[idx[u]];
 #pragma unroll
         for (int j = 0; j < TAPS; ++j)
 #pragma unroll
@@ -116,11 +132,12 @@ rmsnorm_conv_single_kernel(const float* __restrict__ x, int ldx, const float* __
             for (int u = 0; u < 8; ++u) v[j][u] = carried[static_cast<size_t>(j) * C + idx[u]];
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
-            const float h = xv[b][u] * inv * g[u];
+            const float h = MODE == 0 ? xv[b][u] * inv * g[u] : MODE == 1 ? xv[b][u] + yv[b][u] * inv * g[u] : xv[b][u];
             float acc = w[TAPS - 1][u] * h;
 #pragma unroll
             for (int j = 0; j + 1 < TAPS; ++j) acc += w[j][u] * v[j][u];
             if (512 * b + lane + 64 * u < C) {
+                if (MODE == 1) xr[idx[u]] = h;
                 if (write) {
 #pragma unroll
                     for (int j = 1; j + 1 < TAPS; ++j) carried[static_cast<size_t>(j - 1) * C + idx[u]] = v[j][u];
@@ -472,6 +489,30 @@ ssm_chunk_join_kernel(const float* __restrict__ xbc, int ldx, const int* __restr
 
 }  // namespace
 
+// The launch of rmsnorm_conv_single_kernel by taps, width and output type.
+template <int MODE>
+static int stream_conv_single_launch(float* x, int ldx, const float* y, int ldy, const float* wn, float eps, int C, const float* wc,
+                                     int taps, const int* state_slots, float* state, size_t slot_floats, void* out, int ldo,
+                                     int out_dtype, int T, int write, hipStream_t stream) {
+#define RCS(TYPE, TAPS, NB)                                                                                            \
+    rmsnorm_conv_single_kernel<TYPE, 4, TAPS, NB, MODE><<<(T + 3) / 4, 256, 0, stream>>>(x, ldx, y, ldy, wn, eps, C, wc, state_slots, \
+                                                                                        state, slot_floats, static_cast<TYPE*>(out), ldo, T, write)
+#define RCS_NB(TYPE, TAPS)                                                                                             \
+    do { if (C <= 512) RCS(TYPE, TAPS, 1); else if (C <= 1024) RCS(TYPE, TAPS, 2); else RCS(TYPE, TAPS, 4); } while (0)
+#define RCS_TAPS(TYPE)                                                                                                 \
+    switch (taps) {                                                                                                    \
+        case 1: RCS_NB(TYPE, 1); break; case 2: RCS_NB(TYPE, 2); break; case 3: RCS_NB(TYPE, 3); break;                \
+        case 4: RCS_NB(TYPE, 4); break; case 5: RCS_NB(TYPE, 5); break; case 6: RCS_NB(TYPE, 6); break;                \
+        case 7: RCS_NB(TYPE, 7); break; default: RCS_NB(TYPE, 8); break;                                               \
+    }
+    if (out_dtype == MLLM_F32) { RCS_TAPS(float) } else { RCS_TAPS(bf16_t) }
+#undef RCS_TAPS
+#undef RCS_NB
+#undef RCS
+    MLLM_LAUNCH_CHECK();
+    return 0;
+}
+
 extern "C" {
 
 // Convolution + silu of columns [col0, col0 + C) of proj's rows into out [T, C]; then, with `write`, the
@@ -531,23 +572,25 @@ int mllm_rmsnorm_conv_single(const float* x, int ldx, const float* wn, float eps
     if (T <= 0 || C <= 0) return 0;
     if (taps < 1 || taps > 16) return -1;
     if (taps > 8 || C > 2048) return -2;           // sizes this kernel is not made for: norm and convolution apart
-#define RCS(TYPE, TAPS, NB)                                                                                            \
-    rmsnorm_conv_single_kernel<TYPE, 4, TAPS, NB><<<(T + 3) / 4, 256, 0, stream>>>(x, ldx, wn, eps, C, wc, state_slots, state, \
-                                                                                  slot_floats, static_cast<TYPE*>(out), ldo, T, write)
-#define RCS_NB(TYPE, TAPS)                                                                                             \
-    do { if (C <= 512) RCS(TYPE, TAPS, 1); else if (C <= 1024) RCS(TYPE, TAPS, 2); else RCS(TYPE, TAPS, 4); } while (0)
-#define RCS_TAPS(TYPE)                                                                                                 \
-    switch (taps) {                                                                                                    \
-        case 1: RCS_NB(TYPE, 1); break; case 2: RCS_NB(TYPE, 2); break; case 3: RCS_NB(TYPE, 3); break;                \
-        case 4: RCS_NB(TYPE, 4); break; case 5: RCS_NB(TYPE, 5); break; case 6: RCS_NB(TYPE, 6); break;                \
-        case 7: RCS_NB(TYPE, 7); break; default: RCS_NB(TYPE, 8); break;                                               \
-    }
-    if (out_dtype == MLLM_F32) { RCS_TAPS(float) } else { RCS_TAPS(bf16_t) }
-#undef RCS_TAPS
-#undef RCS_NB
-#undef RCS
-    MLLM_LAUNCH_CHECK();
-    return 0;
+    // (this mode only reads x)
+    return stream_conv_single_launch<0>(const_cast<float*>(x), ldx, nullptr, 0, wn, eps, C, wc, taps, state_slots, state, slot_floats, out,
+                                        ldo, out_dtype, T, write, stream);
+}
+
+// For a step of T sequences of one token each, the stream's rows x [T, C] (fp32) and a block's input convolution:
+// with y (a sub-layer's result, fp32 [T, C]) and wn: x += y / sqrt(mean(y^2) + eps) * wn first (x is written), then
+// out = x + conv(x); with y null: out = x + conv(x) alone. Return codes as mllm_rmsnorm_conv_single's.
+int mllm_stream_conv_single(float* x, int ldx, const float* y, int ldy, const float* wn, float eps, int C, const float* wc, int taps,
+                            const int* state_slots, float* state, size_t slot_floats, void* out, int ldo, int out_dtype, int T,
+                            int write, hipStream_t stream) {
+    if (T <= 0 || C <= 0) return 0;
+    if (taps < 1 || taps > 16 || (y != nullptr && wn == nullptr)) return -1;
+    if (taps > 8 || C > 2048) return -2;
+    if (y != nullptr)
+        return stream_conv_single_launch<1>(x, ldx, y, ldy, wn, eps, C, wc, taps, state_slots, state, slot_floats, out, ldo, out_dtype, T,
+                                            write, stream);
+    return stream_conv_single_launch<2>(x, ldx, nullptr, 0, nullptr, eps, C, wc, taps, state_slots, state, slot_floats, out, ldo,
+                                        out_dtype, T, write, stream);
 }
 
 // Tokens of a chunk, rows of n a wavefront keeps, and what the chunks' workspace must hold for a step of T tokens.
