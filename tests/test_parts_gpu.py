@@ -66,6 +66,43 @@ def test_dense_mlp_part(dtype, act):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("experts,top,ff,shared,T", [(5, 2, 24, 40, 9), (3, 3, 16, 0, 70), (1, 1, 32, 8, 1), (12, 1, 8, 16, 33)])
+def test_routed_experts_part(dtype, experts, top, ff, shared, T):
+    """The feed-forward of routed experts alone: joined first and second matrices (the shared expert's columns
+    last), against the plain function token by token. Rows whose router makes a close call are left out in
+    bfloat16 (the part's router reads the bfloat16 input)."""
+    import parts_face as pf
+    import plain_viladra as pv
+    g = torch.Generator().manual_seed(7)
+    D = 48
+    w = {"router": _randn(g, experts, D, std=0.4, dtype=dtype).double()}
+    for e in range(experts):
+        w[f"e{e}.up"] = _randn(g, ff, D, std=0.15, dtype=dtype).double()
+        w[f"e{e}.down"] = _randn(g, D, ff, std=0.15, dtype=dtype).double()
+    names = [f"e{e}." for e in range(experts)]
+    if shared:
+        w["shared.up"] = _randn(g, shared, D, std=0.15, dtype=dtype).double()
+        w["shared.down"] = _randn(g, D, shared, std=0.15, dtype=dtype).double()
+        names.append("shared.")
+    up = torch.cat([w[n + "up"] for n in names], dim=0).to(dtype).to(DEV).contiguous()
+    down = torch.cat([w[n + "down"] for n in names], dim=1).to(dtype).to(DEV).contiguous()
+    part = pf.FeedForward("routed_experts", pf.Params(dtype=pf.DT[dtype], experts=experts, ff=ff, top=top, scale=1.75, activation="relu2",
+                                                      up__weight=up, down__weight=down, router=w["router"].to(dtype).to(DEV)))
+    h = torch.randn(T, D, generator=g).to(dtype)
+    x0 = torch.randn(T, D, generator=g)
+    x = part.forward(h.to(DEV), x0.clone().to(DEV))
+    mlp = {"router": {"experts": experts, "top": top, "scale": 1.75}, "shared": {"ff": shared} if shared else None}
+    ref = x0.double() + pv.routed_experts(h.double(), w, "", mlp)
+    err = (x.cpu().double() - ref).abs().amax(dim=1)
+    if dtype == torch.bfloat16 and top < experts:
+        scores = torch.softmax(h.double() @ w["router"].T, dim=-1).sort(dim=-1, descending=True).values
+        keep = (scores[:, top - 1] - scores[:, top]) > 0.01
+        assert keep.float().mean() > 0.5
+        err = err[keep]
+    assert err.max() <= TOL[dtype] * (4 if dtype == torch.bfloat16 else 1)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_embedding_position_and_head_parts(dtype):
     import parts_face as pf
     g = torch.Generator().manual_seed(2)
