@@ -68,83 +68,82 @@ __global__ void conv_residual_kernel(const float* __restrict__ in, int ld, int C
 }
 
 // A step in which every sequence brings one token: h = x / sqrt(mean(x^2) + eps) * wn and out = h + conv(h) in one
-// kernel, one wavefront per token. The earlier inputs of the convolution are the slot's carried rows, which move up
+// kernel, one workgroup per token. The earlier inputs of the convolution are the slot's carried rows, which move up
 // by one behind the read; h becomes the newest.
-// NB blocks of 512 columns: the row of x stays in registers between the statistics and the convolution. All loads of a
-// block are issued together, without conditions, from clamped (always valid) places, and masked where they are used
-// (a load under a condition, or in a loop of unknown length, is waited for before the next is asked for); TAPS is a
+// NB wavefronts, each with a block of 512 columns: its part of the row stays in registers between the statistics (the
+// wavefronts' sums meet in LDS and are added in the order of the blocks) and the convolution. All loads of a block
+// are issued together, without conditions, from clamped (always valid) places, and masked where they are used (a
+// load under a condition, or in a loop of unknown length, is waited for before the next is asked for); TAPS is a
 // constant for that reason.
 // MODE 0: as above. MODE 1, a norm BEHIND a sub-layer and the next sub-layer's convolution: the stream's row becomes
 // x + y / sqrt(mean(y^2) + eps) * wn (y: the sub-layer's result; x is written back), and h is that row. MODE 2: no norm,
 // h = x.
-template <typename OutT, int WAVES, int TAPS, int NB, int MODE>
-__global__ void __launch_bounds__(64 * WAVES)
+template <typename OutT, int TAPS, int NB, int MODE>
+__global__ void __launch_bounds__(64 * NB)
 rmsnorm_conv_single_kernel(float* x, int ldx, const float* __restrict__ y, int ldy, const float* __restrict__ wn, float eps, int C,
                            const float* __restrict__ wc, const int* __restrict__ state_slots, float* __restrict__ state,
-                           size_t slot_floats, OutT* __restrict__ out, int ldo, int T, int write) {
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MLLM_WAVE), lane = threadIdx.x % MLLM_WAVE;
-    const int t = blockIdx.x * WAVES + wave;
-    if (t >= T) return;
+                           size_t slot_floats, OutT* __restrict__ out, int ldo, int write) {
+    __shared__ float part[NB];
+    const int b = __builtin_amdgcn_readfirstlane(threadIdx.x / MLLM_WAVE), lane = threadIdx.x % MLLM_WAVE;
+    const int t = blockIdx.x;
     const int slot = state_slots[t];
-    if (slot < 0) return;
+    if (slot < 0) return;                      // (the whole workgroup: one token)
     float* xr = x + static_cast<size_t>(t) * ldx;
-    float xv[NB][8], yv[MODE == 1 ? NB : 1][8];
+    int idx[8];
 #pragma unroll
-    for (int b = 0; b < NB; ++b)
+    for (int u = 0; u < 8; ++u) idx[u] = min(512 * b + lane + 64 * u, C - 1);
+    float xv[8], yv[8], g[8], w[TAPS][8], v[TAPS > 1 ? TAPS - 1 : 1][8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) xv[b][u] = xr[min(512 * b + lane + 64 * u, C - 1)];
+    for (int u = 0; u < 8; ++u) xv[u] = xr[idx[u]];
     if (MODE == 1) {
         const float* yr = y + static_cast<size_t>(t) * ldy;
 #pragma unroll
-        for (int b = 0; b < NB; ++b)
-#pragma unroll
-            for (int u = 0; u < 8; ++u) yv[b][u] = yr[min(512 * b + lane + 64 * u, C - 1)];
+        for (int u = 0; u < 8; ++u) yv[u] = yr[idx[u]];
     }
+    const float* carried = state + static_cast<size_t>(slot) * slot_floats;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) g[u] = MODE == 2 ? 1.f : wn[idx[u]];
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j)
+#pragma unroll
+        for (int u = 0; u < 8; ++u) w[j][u] = wc[static_cast<size_t>(idx[u]) * TAPS + j];
+#pragma unroll
+    for (int j = 0; j + 1 < TAPS; ++j)
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[j][u] = carried[static_cast<size_t>(j) * C + idx[u]];
     float inv = 1.f;
     if (MODE != 2) {
         float ss = 0.f;
 #pragma unroll
-        for (int b = 0; b < NB; ++b)
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const float z = MODE == 1 ? yv[b][u] : xv[b][u];
-                ss += (512 * b + lane + 64 * u < C) ? z * z : 0.f;
-            }
-        inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(C) + eps);
-    }
-    float* carried = state + static_cast<size_t>(slot) * slot_floats;
-#pragma unroll
-    for (int b = 0; b < NB; ++b) {
-        if (512 * b >= C) break;
-        int idx[8];
-        float g[8], w[TAPS][8], v[TAPS > 1 ? TAPS - 1 : 1][8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) idx[u] = min(512 * b + lane + 64 * u, C - 1);
-#pragma unroll
-        for (int u = 0; u < 8; ++u) g[u] = MODE == 2 ? 1.f : wn[idx[u]];
-#pragma unroll
-        for (int j = 0; j < TAPS; ++j)
-#pragma unroll
-            for (int u = 0; u < 8; ++u) w[j][u] = wc[static_cast<size_t>(idx[u]) * TAPS + j];
-#pragma unroll
-        for (int j = 0; j + 1 < TAPS; ++j)
-#pragma unroll
-            for (int u = 0; u < 8; ++u) v[j][u] = carried[static_cast<size_t>(j) * C + idx[u]];
-#pragma unroll
         for (int u = 0; u < 8; ++u) {
-            const float h = MODE == 0 ? xv[b][u] * inv * g[u] : MODE == 1 ? xv[b][u] + yv[b][u] * inv * g[u] : xv[b][u];
-            float acc = w[TAPS - 1][u] * h;
+            const float z = MODE == 1 ? yv[u] : xv[u];
+            ss += (512 * b + lane + 64 * u < C) ? z * z : 0.f;
+        }
+        ss = wave_sum(ss);
+        if (NB > 1) {
+            if (lane == 0) part[b] = ss;
+            __syncthreads();
+            ss = 0.f;
 #pragma unroll
-            for (int j = 0; j + 1 < TAPS; ++j) acc += w[j][u] * v[j][u];
-            if (512 * b + lane + 64 * u < C) {
-                if (MODE == 1) xr[idx[u]] = h;
-                if (write) {
+            for (int k = 0; k < NB; ++k) ss += part[k];
+        }
+        inv = 1.0f / sqrtf(ss / static_cast<float>(C) + eps);
+    }
+    float* carried_w = state + static_cast<size_t>(slot) * slot_floats;
 #pragma unroll
-                    for (int j = 1; j + 1 < TAPS; ++j) carried[static_cast<size_t>(j - 1) * C + idx[u]] = v[j][u];
-                    if (TAPS > 1) carried[static_cast<size_t>(TAPS - 2) * C + idx[u]] = h;
-                }
-                out[static_cast<size_t>(t) * ldo + idx[u]] = from_float<OutT>(h + acc);
+    for (int u = 0; u < 8; ++u) {
+        const float h = MODE == 0 ? xv[u] * inv * g[u] : MODE == 1 ? xv[u] + yv[u] * inv * g[u] : xv[u];
+        float acc = w[TAPS - 1][u] * h;
+#pragma unroll
+        for (int j = 0; j + 1 < TAPS; ++j) acc += w[j][u] * v[j][u];
+        if (512 * b + lane + 64 * u < C) {
+            if (MODE == 1) xr[idx[u]] = h;
+            if (write) {
+#pragma unroll
+                for (int j = 1; j + 1 < TAPS; ++j) carried_w[static_cast<size_t>(j - 1) * C + idx[u]] = v[j][u];
+                if (TAPS > 1) carried_w[static_cast<size_t>(TAPS - 2) * C + idx[u]] = h;
             }
+            out[static_cast<size_t>(t) * ldo + idx[u]] = from_float<OutT>(h + acc);
         }
     }
 }
@@ -495,10 +494,13 @@ static int stream_conv_single_launch(float* x, int ldx, const float* y, int ldy,
                                      int taps, const int* state_slots, float* state, size_t slot_floats, void* out, int ldo,
                                      int out_dtype, int T, int write, hipStream_t stream) {
 #define RCS(TYPE, TAPS, NB)                                                                                            \
-    rmsnorm_conv_single_kernel<TYPE, 4, TAPS, NB, MODE><<<(T + 3) / 4, 256, 0, stream>>>(x, ldx, y, ldy, wn, eps, C, wc, state_slots, \
-                                                                                        state, slot_floats, static_cast<TYPE*>(out), ldo, T, write)
+    rmsnorm_conv_single_kernel<TYPE, TAPS, NB, MODE><<<T, 64 * NB, 0, stream>>>(x, ldx, y, ldy, wn, eps, C, wc, state_slots, state, \
+                                                                               slot_floats, static_cast<TYPE*>(out), ldo, write)
 #define RCS_NB(TYPE, TAPS)                                                                                             \
-    do { if (C <= 512) RCS(TYPE, TAPS, 1); else if (C <= 1024) RCS(TYPE, TAPS, 2); else RCS(TYPE, TAPS, 4); } while (0)
+    do {                                                                                                               \
+        if (C <= 512) RCS(TYPE, TAPS, 1); else if (C <= 1024) RCS(TYPE, TAPS, 2); else if (C <= 1536) RCS(TYPE, TAPS, 3);   \
+        else RCS(TYPE, TAPS, 4);                                                                                       \
+    } while (0)
 #define RCS_TAPS(TYPE)                                                                                                 \
     switch (taps) {                                                                                                    \
         case 1: RCS_NB(TYPE, 1); break; case 2: RCS_NB(TYPE, 2); break; case 3: RCS_NB(TYPE, 3); break;                \
