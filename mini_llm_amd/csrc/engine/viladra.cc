@@ -14,6 +14,8 @@
 //              {"type": "gla", "mixer": {"heads", "dim", "vdim", "tau"}, "mlp": ...},
 //              {"type": "attention", "mixer": {"heads", "kv_heads", "dim", "vdim", "scale", "mask": {"size"}}, "mlp": ...}]}
 //   mlp: {"kind": "moe", "router": {"experts", "top", "scale"}, "expert": {"ff"}, "shared": {"ff"} | null} | null
+//   May be absent: canon, embedding, logit_softcap, rot (none of it), kv_heads (as many as heads), vdim (as wide as dim),
+//   mlp.kind, router.scale (1), mlp.shared, mlp.
 // Tensors: embed, l<i>.norm1[/norm2], l<i>.canon1[/canon2], l<i>.dwa, l<i>.mix.*, l<i>.mlp.{router, e<k>.up, e<k>.down,
 // shared.up, shared.down}, final.norm; linear weights are stored [out, in]. The rank of a gla layer's decay map is
 // not in config.json: it is the height of the stored l<i>.mix.a1.
@@ -101,7 +103,8 @@ struct ViladraConfig {
             const Json& m = need_object(l, "mixer", where);
             LayerConfig lc;
             MixerConfig& x = lc.mix;
-            x.heads = need_int(m, "heads", where); x.dim = need_int(m, "dim", where); x.vdim = need_int(m, "vdim", where);
+            x.heads = need_int(m, "heads", where); x.dim = need_int(m, "dim", where);
+            x.vdim = m.find("vdim") != nullptr ? need_int(m, "vdim", where) : x.dim;          // (no vdim: values as wide as keys)
             if (type->string() == "retention") {
                 x.kind = MixerConfig::Retention;
                 const Json* dec = m.find("decay");
@@ -128,7 +131,7 @@ struct ViladraConfig {
                 if (const Json* r = m.find("rank")) if (r->is_integer() && r->integer() >= 1) x.rank = r->integer();
             } else if (type->string() == "attention") {
                 x.kind = MixerConfig::Attention;
-                x.kv_heads = need_int(m, "kv_heads", where);
+                x.kv_heads = m.find("kv_heads") != nullptr ? need_int(m, "kv_heads", where) : x.heads;     // (none: no grouping)
                 if (x.heads % x.kv_heads != 0) throw ConfigError("config.json: " + where + "heads is not a multiple of kv_heads");
                 x.scale = need_num(m, "scale", where);
                 x.mask = need_int(need_object(m, "mask", where), "size", where + "mask: ");
@@ -139,7 +142,7 @@ struct ViladraConfig {
             if (mlp != nullptr && !mlp->is_null()) {
                 if (!mlp->is_object()) throw ConfigError("config.json: " + where + "'mlp' must be an object or null");
                 const Json* kind = mlp->find("kind");
-                if (kind == nullptr || !kind->is_string() || kind->string() != "moe")
+                if (kind != nullptr && (!kind->is_string() || kind->string() != "moe"))
                     throw ConfigError("config.json: " + where + "mlp.kind must be 'moe'");
                 MlpConfig& f = lc.mlp;
                 f.present = true;

@@ -40,6 +40,18 @@ def test_registered_and_tensors_follow_the_layer_list():
     assert free["l0.mix.a1"] == 0 and free["l0.mix.a2"] == 1 and free["l0.mix.q"] is None
 
 
+def test_keys_that_may_be_absent_have_the_plain_meaning():
+    """No kv_heads: as many key/value heads as heads; no vdim: values as wide as keys; no mlp.kind: routed experts."""
+    cfg = copy.deepcopy(vc.MIXED_A)
+    att = cfg["layers"][1]["mixer"]
+    heads, dim = att["heads"], att["dim"]
+    att.pop("kv_heads"); att.pop("vdim")
+    cfg["layers"][0]["mlp"].pop("kind")
+    shapes = {t["name"]: t["shape"] for t in describe_config(cfg)["tensors"]}
+    assert shapes["l1.mix.k"] == [heads * dim, cfg["width"]] and shapes["l1.mix.v"] == [heads * dim, cfg["width"]]
+    assert "l0.mlp.router" in shapes
+
+
 @pytest.mark.parametrize("change, message", [
     (lambda c: c["layers"][1].__setitem__("type", "lstm"), "unknown layer type"),
     (lambda c: c["layers"][1]["mixer"].__setitem__("kv_heads", 3), "multiple of kv_heads"),
