@@ -67,6 +67,62 @@ __global__ void conv_residual_kernel(const float* __restrict__ in, int ld, int C
     out[static_cast<size_t>(t) * ldo + ch] = from_float<OutT>(own + acc);
 }
 
+// The same four channels a thread (16-byte loads; the rows' widths and the places are multiples of four floats). A
+// token with taps - 1 tokens of its own portion in front of it reads them all from `in`, without conditions, so its
+// loads are in flight together; the first tokens of a portion read the slot's carried rows where the portion has none.
+// A wavefront holds one token's channels (or the border of two tokens), so the two ways seldom meet in one.
+__device__ __forceinline__ void store4(float* p, const float (&v)[4]) { *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]); }
+__device__ __forceinline__ void store4(bf16_t* p, const float (&v)[4]) {
+    *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+}
+template <typename OutT, int TAPS>
+__global__ void conv_residual_vec_kernel(const float* __restrict__ in, int ld, int C, const float* __restrict__ w,
+                                         const int* __restrict__ token_seq, const int* __restrict__ cu_q,
+                                         const int* __restrict__ state_slots, float* __restrict__ state, size_t slot_floats,
+                                         OutT* __restrict__ out, int ldo, long long total4, int carry) {
+    const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= total4) return;
+    const int C4 = C / 4;
+    const int t = static_cast<int>(i / C4), ch = static_cast<int>(i % C4) * 4;
+    const int b = token_seq[t], slot = state_slots[b];
+    if (slot < 0) return;
+    const int first = cu_q[b], k = t - first;
+    float* carried = state + static_cast<size_t>(slot) * slot_floats;
+    float4 wf[TAPS], v[TAPS];             // wf: the four channels' taps one behind the other (4 * TAPS floats)
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) wf[j] = *reinterpret_cast<const float4*>(w + static_cast<size_t>(ch) * TAPS + 4 * j);
+    if (k >= TAPS - 1) {
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) v[j] = *reinterpret_cast<const float4*>(in + static_cast<size_t>(t - (TAPS - 1 - j)) * ld + ch);
+    } else {
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) {
+            const int idx = k - (TAPS - 1 - j);
+            v[j] = idx >= 0 ? *reinterpret_cast<const float4*>(in + static_cast<size_t>(first + idx) * ld + ch)
+                            : *reinterpret_cast<const float4*>(carried + static_cast<size_t>(TAPS - 1 + idx) * C + ch);
+        }
+    }
+    float wv[4 * TAPS];
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) { wv[4 * j] = wf[j].x; wv[4 * j + 1] = wf[j].y; wv[4 * j + 2] = wf[j].z; wv[4 * j + 3] = wf[j].w; }
+    float r[4] = {v[TAPS - 1].x, v[TAPS - 1].y, v[TAPS - 1].z, v[TAPS - 1].w};
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) {
+        acc[0] += wv[0 * TAPS + j] * v[j].x;
+        acc[1] += wv[1 * TAPS + j] * v[j].y;
+        acc[2] += wv[2 * TAPS + j] * v[j].z;
+        acc[3] += wv[3 * TAPS + j] * v[j].w;
+    }
+    if (carry) {
+#pragma unroll
+        for (int j = 1; j < TAPS; ++j) *reinterpret_cast<float4*>(carried + static_cast<size_t>(j - 1) * C + ch) = v[j];
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) r[q] += acc[q];
+    store4(out + static_cast<size_t>(t) * ldo + ch, r);
+}
+
 // A step in which every sequence brings one token: h = x / sqrt(mean(x^2) + eps) * wn and out = h + conv(h) in one
 // kernel, one workgroup per token. The earlier inputs of the convolution are the slot's carried rows, which move up
 // by one behind the read; h becomes the newest.
@@ -549,13 +605,32 @@ int mllm_conv_residual(const float* in, int ld, int C, const float* w, int taps,
     if (taps < 1 || taps > 16) return -1;
     const long long total = static_cast<long long>(T) * C;
     const bool single = T == B && write && taps > 1;
-    const int blocks = static_cast<int>((total + 255) / 256);
-    if (out_dtype == MLLM_F32)
-        conv_residual_kernel<float><<<blocks, 256, 0, stream>>>(in, ld, C, w, taps, token_seq, cu_q, state_slots, state, slot_floats,
-                                                                static_cast<float*>(out), ldo, total, single ? 1 : 0);
-    else
-        conv_residual_kernel<bf16_t><<<blocks, 256, 0, stream>>>(in, ld, C, w, taps, token_seq, cu_q, state_slots, state, slot_floats,
-                                                                 static_cast<bf16_t*>(out), ldo, total, single ? 1 : 0);
+    const bool vec = taps <= 8 && C % 4 == 0 && ld % 4 == 0 && ldo % 4 == 0 && slot_floats % 4 == 0 &&
+                     ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(state) |
+                       reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+    if (vec) {
+        const long long total4 = total / 4;
+        const int blocks4 = static_cast<int>((total4 + 255) / 256);
+#define CRV(TYPE, TAPS)                                                                                                \
+    conv_residual_vec_kernel<TYPE, TAPS><<<blocks4, 256, 0, stream>>>(in, ld, C, w, token_seq, cu_q, state_slots, state, slot_floats, \
+                                                                     static_cast<TYPE*>(out), ldo, total4, single ? 1 : 0)
+#define CRV_TAPS(TYPE)                                                                                                 \
+    switch (taps) {                                                                                                    \
+        case 1: CRV(TYPE, 1); break; case 2: CRV(TYPE, 2); break; case 3: CRV(TYPE, 3); break; case 4: CRV(TYPE, 4); break; \
+        case 5: CRV(TYPE, 5); break; case 6: CRV(TYPE, 6); break; case 7: CRV(TYPE, 7); break; default: CRV(TYPE, 8); break; \
+    }
+        if (out_dtype == MLLM_F32) { CRV_TAPS(float) } else { CRV_TAPS(bf16_t) }
+#undef CRV_TAPS
+#undef CRV
+    } else {
+        const int blocks = static_cast<int>((total + 255) / 256);
+        if (out_dtype == MLLM_F32)
+            conv_residual_kernel<float><<<blocks, 256, 0, stream>>>(in, ld, C, w, taps, token_seq, cu_q, state_slots, state, slot_floats,
+                                                                    static_cast<float*>(out), ldo, total, single ? 1 : 0);
+        else
+            conv_residual_kernel<bf16_t><<<blocks, 256, 0, stream>>>(in, ld, C, w, taps, token_seq, cu_q, state_slots, state,
+                                                                     slot_floats, static_cast<bf16_t*>(out), ldo, total, single ? 1 : 0);
+    }
     MLLM_LAUNCH_CHECK();
     if (write && taps > 1 && !single) {
         const long long pairs = static_cast<long long>(B) * C;
