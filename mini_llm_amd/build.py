@@ -78,7 +78,7 @@ LIBRARIES: Dict[str, dict] = {
         "kind": "hiphost",
         "sources": ["engine/ops.cc", "engine/ops_sequence.cc", "engine/ops_scored.cc", "engine/parts.cc", "engine/parts_gated.cc",
                     "engine/mamba2.cc", "engine/latent_attention.cc", "engine/scored_attention.cc", "engine/recurrent_parts.cc", "engine/linear_attention.cc", "engine/json.cc", "engine/weights.cc", "engine/arch.cc",
-                    "engine/gpt2.cc", "engine/kugulorn.cc", "engine/rekirax.cc", "engine/viladra.cc", "engine/engine.cc", "engine/engine_api.cc"],
+                    "engine/gpt2.cc", "engine/kugulorn.cc", "engine/rekirax.cc", "engine/viladra.cc", "engine/sunulorn.cc", "engine/engine.cc", "engine/engine_api.cc"],
         "headers": ["kernels/score_shape.h", "engine/ops.h", "engine/parts.h", "engine/kernels.h", "engine/json.h", "engine/weights.h",
                     "engine/arch.h", "engine/engine.h", "runtime/cache_manager.h", "runtime/scheduler.h"],
         "needs": ["elementwise", "gemm_f32", "gemm_bf16", "attention", "attention_decode", "attention_prefill",

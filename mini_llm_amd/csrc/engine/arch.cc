@@ -22,6 +22,7 @@ void register_builtin_architectures() {
         register_kugulorn();
         register_rekirax();
         register_viladra();
+        register_sunulorn();
         if (const char* env = std::getenv("MINI_LLM_PLUGINS")) {
             std::stringstream ss(env);
             for (std::string path; std::getline(ss, path, ':');)

@@ -51,6 +51,7 @@ void register_gpt2();              // gpt2.cc
 void register_kugulorn();          // kugulorn.cc
 void register_rekirax();           // rekirax.cc
 void register_viladra();           // viladra.cc
+void register_sunulorn();          // sunulorn.cc
 // Loads a shared library whose initialisers register parts and architectures (dlopen; stays loaded).
 // Also called for every path in the environment variable MINI_LLM_PLUGINS (colon-separated), once.
 void load_plugin(const std::string& path);

@@ -34,13 +34,14 @@ CacheStorage::CacheStorage(const std::vector<CacheNeed>& needs, int page_size, i
 
 void CacheStorage::allocate(const std::vector<CacheNeed>& needs, int n_pages, int n_state_slots) {
     const int page_size = page_size_, dtype = dtype_;
-    struct Key { int hkv, hd, vd, window; bool operator==(const Key& o) const { return hkv == o.hkv && hd == o.hd && vd == o.vd && window == o.window; } };
+    struct Key { int hkv, hd, vd, window, keep; bool operator==(const Key& o) const { return hkv == o.hkv && hd == o.hd && vd == o.vd && window == o.window && keep == o.keep; } };
     std::vector<Key> keys;
     std::vector<std::vector<int>> members;
     std::vector<int> group_of(needs.size(), -1);
     for (size_t c = 0; c < needs.size(); ++c) {
         if (!(needs[c].kind & 1)) continue;
-        const Key k{needs[c].n_kv_heads, needs[c].head_dim, needs[c].value_dim < 0 ? needs[c].head_dim : needs[c].value_dim, needs[c].window};
+        const Key k{needs[c].n_kv_heads, needs[c].head_dim, needs[c].value_dim < 0 ? needs[c].head_dim : needs[c].value_dim, needs[c].window,
+                    needs[c].window > 0 ? needs[c].keep_first : 0};
         size_t g = 0;
         while (g < keys.size() && !(keys[g] == k)) ++g;
         if (g == keys.size()) { keys.push_back(k); members.emplace_back(); }
@@ -54,6 +55,7 @@ void CacheStorage::allocate(const std::vector<CacheNeed>& needs, int n_pages, in
         gs.page_size = page_size;
         gs.n_pages = n_pages;
         gs.window = keys[g].window;
+        gs.keep_first = keys[g].keep;
         group_specs_.push_back(gs);
         const int64_t rows = static_cast<int64_t>(n_pages) * page_size, kv_dim = static_cast<int64_t>(keys[g].hkv) * keys[g].hd;
         const int64_t v_dim = static_cast<int64_t>(keys[g].hkv) * keys[g].vd;         // 0: key rows only

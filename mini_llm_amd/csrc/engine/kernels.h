@@ -84,7 +84,7 @@ int mllm_fill_zero(void* p, size_t bytes, hipStream_t stream);
 // ssm.hip
 int mllm_conv_silu(const float* proj, int ld, int col0, int C, const float* w, const float* bias, int taps,
                    const int* token_seq, const int* cu_q, const int* state_slots, float* state, size_t slot_floats,
-                   float* out, int ldo, int T, int B, int write, hipStream_t stream);
+                   float* out, int ldo, int T, int B, int write, hipStream_t stream, int activation = 1);
 int mllm_conv_residual(const float* in, int ld, int C, const float* w, int taps, const int* token_seq, const int* cu_q,
                        const int* state_slots, float* state, size_t slot_floats, void* out, int ldo, int out_dtype, int T,
                        int B, int write, hipStream_t stream);
@@ -121,12 +121,13 @@ int mllm_latent_expand(const void* o_lat, int ldo, const void* w_uv, int ldw, vo
 int mllm_qk_prepare(const float* proj, int ld, int q_col, int k_col, int v_col, int T, int H, int G, int d, int dv,
                     int norm_mode, const float* wq, const float* wk, float eps, int rot_dims, double rot_base,
                     const int* positions, const int* slots, void* q_out, int ldq, void* k_pages, void* v_pages, int dtype,
-                    hipStream_t stream);
+                    hipStream_t stream, int interleaved = 0);
 int mllm_scored_attention_rows(const void* q, int ldq, const void* k_pages, const void* v_pages, const int* block_tables,
                                int max_blocks, const int* token_seq, const int* positions, int n_tokens, int H, int G, int d,
                                int dv, int page_size, float scale, float softcap, int window, int chunk, const float* r1,
                                const float* r2, const float* gate, int ldg, void* out, int ldo, int dtype, hipStream_t stream,
-                               int sigmoid_weights = 0, const float* score_bias = nullptr, int gate_per_head = 0);
+                               int sigmoid_weights = 0, const float* score_bias = nullptr, int gate_per_head = 0,
+                               const float* slope = nullptr, const float* sink = nullptr, int keep_first = 0);
 
 int mllm_gate_mul(void* x, int ldx, const float* gate, int ldg, int T, int N, int dtype, hipStream_t stream);
 
@@ -152,6 +153,9 @@ int mllm_glu_act(const void* gu, int ld, int T, int F, int act, void* out, int l
 // moe.hip
 int mllm_moe_act(const void* up, int ldu, const float* logits, int ldl, int E, int ff, int shared_ff, int top, float scale, void* out, int ldo,
                  float* weights_out, int ldw, int T, int dtype, hipStream_t stream);
+int mllm_moe_glu_act(const void* up, int ldu, const float* logits, int ldl, int E, int ff, int shared_ff, int top, float scale,
+                     int sigmoid_router, float limit, float shared_limit, float alpha, int weight_on_input, int shared_gate, void* out,
+                     int ldo, int T, int dtype, hipStream_t stream);
 
 // sampling.hip
 int mllm_argmax_chunks(int V);

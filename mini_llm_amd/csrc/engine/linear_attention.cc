@@ -134,29 +134,56 @@ private:
 // A mixture of small feed-forward experts beside an optional shared one:
 //   y = sum_(e chosen) w_e W_down,e act(W_up,e h) + W_down,s act(W_up,s h),   act(z) = relu(z)^2
 // The router's logits W_r h are a product of their own with fp32 results (its operands are the compute dtype's: a
-// checkpoint's bfloat16 router is held exactly), their softmax over all experts is fp32; the `top` experts with the
-// largest scores are chosen (the lower index wins a tie) and w_e = scale * score_e, not renormalised. The experts' first products are one
+// checkpoint's bfloat16 router is held exactly); the scores are their softmax over all experts, or (router "sigmoid")
+// every logit's sigmoid on its own, in fp32; the `top` experts with the largest scores are chosen (the lower index
+// wins a tie) and w_e = scale * score_e, not renormalised. The experts' first products are one
 // joined product (up.weight rows [expert 0 | expert 1 | ... | shared]), the activation multiplies every expert's
 // block by w_e (zero for an expert that was not chosen), and the second products are one joined product too
 // (down.weight columns in the same order).
-// Parameters: dtype, experts, ff (an expert's hidden width), top, scale; tensors router [experts, width],
-// up.weight [experts * ff + shared_ff, width], down.weight [width, experts * ff + shared_ff].
+// With the activation "clamped_glu" an expert is gated and clamped,
+//   expert(h) = W_down (g sigmoid(alpha g) (u + 1)),  g = min(W_gate h, limit),  u = clamp(W_up h, -limit, limit),
+// up.weight's rows are [expert 0: gate | up] ... [shared: gate | up] (ff rows each; the shared expert shared_ff, with a
+// limit of its own), and with weight_on_input the weight multiplies what the expert READS, y = sum_e expert_e(w_e h):
+// the gate's and the up's products are linear, so the activation scales them before it clamps. With shared_gate the
+// router's matrix has one more row, and the shared expert's result is multiplied by the sigmoid of that logit.
+// Parameters: dtype, experts, ff (an expert's hidden width), top, scale, strings activation, router (softmax);
+// clamped_glu: limit, shared_limit, alpha, weight_on_input, shared_gate; tensors router [experts (+ 1), width],
+// up.weight [experts * ff + shared_ff (clamped_glu: twice that), width], down.weight [width, experts * ff + shared_ff].
 class RoutedExperts final : public FeedForward {
 public:
     explicit RoutedExperts(const Params& p) {
         dtype_ = p.integer("dtype");
-        E_ = p.integer("experts"); ff_ = p.integer("ff"); top_ = p.integer("top");
-        scale_ = static_cast<float>(p.number("scale", 1.0));
+        glu_.experts = E_ = p.integer("experts"); glu_.ff = ff_ = p.integer("ff"); glu_.top = top_ = p.integer("top");
+        glu_.scale = scale_ = static_cast<float>(p.number("scale", 1.0));
         const std::string& act = p.string("activation");
-        if (act != "relu2") fail("routed_experts: unknown activation '%s' (known: relu2)", act.c_str());
+        if (act == "clamped_glu") gated_ = true;
+        else if (act != "relu2") fail("routed_experts: unknown activation '%s' (known: relu2, clamped_glu)", act.c_str());
+        if (p.str.count("router")) {
+            const std::string& r = p.string("router");
+            if (r == "sigmoid") glu_.sigmoid_router = true;
+            else if (r != "softmax") fail("routed_experts: unknown router '%s' (known: softmax, sigmoid)", r.c_str());
+        }
+        if (glu_.sigmoid_router && !gated_) fail("routed_experts: sigmoid scores go with the clamped_glu activation");
         up_ = Linear(p.weights("up.weight"), nullptr);
         down_ = Linear(p.weights("down.weight"), nullptr);
         router_ = Linear(p.weights("router"), nullptr);
         if (E_ < 1 || ff_ < 1 || top_ < 1 || top_ > E_) fail("routed_experts: %d of %d experts of %d do not fit", top_, E_, ff_);
-        if (router_.out_features() != E_ || router_.in_features() != up_.in_features())
-            fail("routed_experts: the router must be [%d, %d]", E_, up_.in_features());
-        if (up_.out_features() < E_ * ff_ || down_.in_features() != up_.out_features() || down_.out_features() != up_.in_features())
+        if (gated_) {
+            glu_.limit = static_cast<float>(p.number("limit"));
+            glu_.alpha = static_cast<float>(p.number("alpha", 1.0));
+            glu_.weight_on_input = p.number("weight_on_input", 0) != 0;
+            glu_.shared_gate = p.number("shared_gate", 0) != 0;
+            glu_.shared_ff = down_.in_features() - E_ * ff_;
+            glu_.shared_limit = glu_.shared_ff > 0 ? static_cast<float>(p.number("shared_limit")) : 0.f;
+            if (!(glu_.limit > 0.f) || (glu_.shared_ff > 0 && !(glu_.shared_limit > 0.f))) fail("routed_experts: the limits must be positive");
+            if (glu_.shared_ff < 0 || up_.out_features() != 2 * down_.in_features() || (glu_.shared_gate && glu_.shared_ff == 0))
+                fail("routed_experts: the joined products' shapes do not fit %d gated experts of %d", E_, ff_);
+        } else if (up_.out_features() < E_ * ff_ || down_.in_features() != up_.out_features()) {
             fail("routed_experts: the joined products' shapes do not fit %d experts of %d", E_, ff_);
+        }
+        if (router_.out_features() != E_ + (glu_.shared_gate ? 1 : 0) || router_.in_features() != up_.in_features())
+            fail("routed_experts: the router must be [%d, %d]", E_ + (glu_.shared_gate ? 1 : 0), up_.in_features());
+        if (down_.out_features() != up_.in_features()) fail("routed_experts: the second products must lead back to the width");
     }
     void forward(NormedInput& h, const StepView& step, const Tensor2& x, Arena& arena, hipStream_t s) const override {
         run(h, step, x, arena, s, ADD_RESIDUAL);
@@ -165,21 +192,27 @@ public:
         run(h, step, x, arena, s, STORE_F32);
     }
     void run(NormedInput& h, const StepView& step, const Tensor2& x, Arena& arena, hipStream_t s, int out_epilogue) const {
-        const int T = step.n_tokens, N = up_.out_features();
+        const int T = step.n_tokens, N = up_.out_features(), R = router_.out_features();
         const Tensor2& in = h.tensor(arena, s);
-        const int lde = (E_ + 3) / 4 * 4;
-        Tensor2 logits(arena.take(static_cast<size_t>(T) * lde * 4), F32, T, E_, lde);
+        const int lde = (R + 3) / 4 * 4;
+        Tensor2 logits(arena.take(static_cast<size_t>(T) * lde * 4), F32, T, R, lde);
         router_(in, logits, STORE_F32, nullptr, s);
         StageTimes::get().mark("router", s);
         Tensor2 inner = arena.tensor(dtype_, T, N);
         up_(in, inner, STORE, nullptr, s);
         StageTimes::get().mark("fc1", s);
-        moe_act(inner, logits, ff_, top_, scale_, inner, nullptr, s);            // in place
-        down_(inner, x, out_epilogue, nullptr, s);
+        if (gated_) {
+            Tensor2 act = arena.tensor(dtype_, T, down_.in_features());
+            moe_glu_act(inner, logits, glu_, act, s);
+            down_(act, x, out_epilogue, nullptr, s);
+        } else {
+            moe_act(inner, logits, ff_, top_, scale_, inner, nullptr, s);            // in place
+            down_(inner, x, out_epilogue, nullptr, s);
+        }
         StageTimes::get().mark("fc2", s);
     }
     size_t workspace_bytes(int tokens) const override {
-        return static_cast<size_t>(tokens) * ((up_.out_features() + up_.in_features()) * dtype_size(dtype_) + (E_ + 4) * 4) + 2048;
+        return static_cast<size_t>(tokens) * ((up_.out_features() + down_.in_features() + up_.in_features()) * dtype_size(dtype_) + (E_ + 8) * 4) + 2048;
     }
     void reserve(int, hipStream_t s) const override { reserve_linear_scratch(s); }
     void add_cost(StepCost& c) const override {
@@ -191,6 +224,8 @@ public:
 private:
     int dtype_ = BF16, E_ = 0, ff_ = 0, top_ = 0;
     float scale_ = 1.f;
+    bool gated_ = false;
+    MoeGlu glu_;
     Linear up_, down_, router_;
 };
 

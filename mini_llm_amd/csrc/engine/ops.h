@@ -24,6 +24,8 @@ inline size_t dtype_size(int dt) { return dt == F32 ? 4 : 2; }
 const char* dtype_name(int dt);
 
 enum Epilogue : int { STORE = 0, GELU_TANH = 1, GELU_ERF = 2, ADD_RESIDUAL = 3, STORE_F32 = 4 };
+// Activations that only the gated feed-forward's kernel knows (glu_act), beside GELU_TANH.
+enum GluActivation : int { GLU_SILU = 5 };
 
 class OpError : public std::runtime_error {
 public:
@@ -194,8 +196,9 @@ struct StateArgs {
 };
 // out[t, :] = silu(conv(columns [col0, col0 + C) of proj)), causal per sequence over `taps` inputs, the inputs
 // before a portion taken from the slot's first (taps - 1) * C floats, which are brought up to date afterwards.
+// With `silu` false the convolution stands alone: no activation, and the bias may be null.
 void conv_silu(const Tensor2& proj, int col0, const Tensor2& weight, const float* bias, const StateArgs& st,
-               const Tensor2& out, hipStream_t stream);
+               const Tensor2& out, hipStream_t stream, bool silu = true);
 // The Mamba-2 scan (kernels/ssm.hip) over xbc [T, H*P + 2*G*N] and the raw step sizes (columns dt_col.. of
 // proj), state at `scan_offset` floats into the slot. y comes as ssm_scan_parts(N) shares, each [T, H*P] fp32
 // and y.rows * y.stride floats after the one before (y is the first); their sum in the order of their index is
@@ -269,11 +272,16 @@ struct ScoredShape {
     int window = 0, chunk = 0;                 // sliding window or chunked causal mask; both 0: plain causal
     const float* r1 = nullptr;                 // per head: s -= r1 ln(1 + r2 (i - j)); null: none
     const float* r2 = nullptr;
-    int norm_mode = 0;                         // 0 none, 1 per head with one weight [dim], 2 over the whole row
+    int keep_first = 0;                        // with a window: the sequence's first keep_first positions stay visible too
+    const float* slope = nullptr;              // per head: s -= slope (i - j) (instead of r1, r2); null: none
+    const float* sink = nullptr;               // per head: one more term exp(sink) in the softmax's denominator; null: none
+    int norm_mode = 0;                         // 0 none, 1 per head with one weight [dim], 2 over the whole row,
+                                               // 3 every head to unit root mean square BEHIND the rotation, no weight
     const float* q_norm = nullptr;
     const float* k_norm = nullptr;
     float eps = 1e-6f;
-    int rot_dims = 0;                          // the first rot_dims columns of a head are turned (half-split pairs)
+    int rot_dims = 0;                          // the first rot_dims columns of a head are turned (half-split pairs,
+    bool rot_interleaved = false;              // or with rot_interleaved column 2i with column 2i + 1)
     double rot_base = 10000.0;
     // weights without a softmax: a visible key's weight is sigmoid(score + score_bias[h]) (score_bias per head, or
     // null), not normalised over the keys
@@ -283,7 +291,8 @@ struct ScoredShape {
 };
 // From the fp32 rows of the input projection (queries at q_col, keys at k_col, values at v_col; v_col < 0: the
 // values are the keys before their norm): q [T, heads * dim] normed and turned, and the keys and values written
-// to their page rows (slots[t]).
+// to their page rows (slots[t]). k_col < 0: queries only (the keys and values are another layer's; the pages are
+// not touched and may be empty tensors).
 void qk_prepare(const Tensor2& proj, int q_col, int k_col, int v_col, const ScoredShape& sh, const int* positions,
                 const int* slots, const Tensor2& q, const Tensor2& k_pages, const Tensor2& v_pages, hipStream_t stream);
 struct ScoredStep {
@@ -343,10 +352,18 @@ void depth_mix(const Tensor2& x, const Tensor2& kept, int n_old, const float* w,
 // shared expert's) are relu(.)^2 alone. out may be up. `weights` (optional, [T, E] fp32) receives the weights.
 void moe_act(const Tensor2& up, const Tensor2& logits, int ff, int top, float scale, const Tensor2& out, const Tensor2* weights,
              hipStream_t stream);
+// The routed experts' activation for gated, clamped experts (kernels/moe.hip): up [T, 2 (E ff + shared_ff)] with rows
+// [expert: gate | up] ... [shared: gate | up], logits [T, E (+ 1: the shared expert's gate)] fp32, out [T, E ff + shared_ff].
+struct MoeGlu {
+    int experts = 0, ff = 0, shared_ff = 0, top = 0;
+    float scale = 1.f, limit = 0.f, shared_limit = 0.f, alpha = 1.f;
+    bool sigmoid_router = false, weight_on_input = false, shared_gate = false;
+};
+void moe_glu_act(const Tensor2& up, const Tensor2& logits, const MoeGlu& m, const Tensor2& out, hipStream_t stream);
 
 // out = [a | b] row by row in out's dtype (a, b fp32 [T, D])
 void concat_cast(const Tensor2& a, const Tensor2& b, const Tensor2& out, hipStream_t stream);
-// out[t, j] = act(gu[t, j]) * gu[t, F + j] (act: GELU_TANH)
+// out[t, j] = act(gu[t, j]) * gu[t, F + j] (act: GELU_TANH or GLU_SILU)
 void glu_act(const Tensor2& gu, int act, const Tensor2& out, hipStream_t stream);
 
 // `mirror` (optional): a second place for the chosen tokens, which may be pinned host memory (the kernel that

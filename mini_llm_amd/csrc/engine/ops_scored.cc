@@ -34,6 +34,9 @@ void check_shape(const ScoredShape& sh, const char* what) {
         fail("%s: %d heads over %d key/value heads of %d / %d do not fit", what, sh.n_heads, sh.n_kv_heads, sh.dim, sh.value_dim);
     if (sh.window < 0 || sh.chunk < 0 || (sh.window > 0 && sh.chunk > 0)) fail("%s: a window or a chunk, not both", what);
     if ((sh.r1 != nullptr) != (sh.r2 != nullptr)) fail("%s: the distance bias needs both of its numbers per head", what);
+    if (sh.slope != nullptr && sh.r1 != nullptr) fail("%s: a linear or a logarithmic distance bias, not both", what);
+    if (sh.sink != nullptr && sh.sigmoid_weights) fail("%s: a sink stands in a softmax's denominator; sigmoid weights have none", what);
+    if (sh.keep_first < 0 || (sh.keep_first > 0 && sh.window <= 0)) fail("%s: kept first positions go with a sliding window", what);
 }
 }  // namespace
 
@@ -111,21 +114,29 @@ void qk_prepare(const Tensor2& proj, int q_col, int k_col, int v_col, const Scor
     need_act(q, "qk_prepare: q");
     const int64_t nq = static_cast<int64_t>(sh.n_heads) * sh.dim, nk = static_cast<int64_t>(sh.n_kv_heads) * sh.dim,
                   nv = static_cast<int64_t>(sh.n_kv_heads) * sh.value_dim;
-    if (q_col < 0 || q_col + nq > proj.cols || k_col < 0 || k_col + nk > proj.cols || (v_col >= 0 && v_col + nv > proj.cols))
+    const bool keys = k_col >= 0;
+    if (q_col < 0 || q_col + nq > proj.cols || (keys && k_col + nk > proj.cols) || (keys && v_col >= 0 && v_col + nv > proj.cols))
         fail("qk_prepare: queries, keys or values lie outside the projection's rows of %lld", (long long)proj.cols);
-    if (v_col < 0 && sh.value_dim != sh.dim) fail("qk_prepare: values taken from the keys must have the keys' width");
+    if (keys && v_col < 0 && sh.value_dim != sh.dim) fail("qk_prepare: values taken from the keys must have the keys' width");
     if (q.rows != proj.rows || q.cols != nq) fail("qk_prepare: q must be [T, %lld]", (long long)nq);
+    if (!keys) {
+        if (sh.norm_mode == 2) fail("qk_prepare: a norm over the whole row needs the keys");
+        check(mllm_qk_prepare(static_cast<const float*>(proj.data), i32(proj.stride), q_col, 0, 0, i32(proj.rows), sh.n_heads, 0,
+                              sh.dim, sh.value_dim, sh.norm_mode, sh.q_norm, sh.q_norm, sh.eps, sh.rot_dims, sh.rot_base, positions, nullptr, q.data,
+                              i32(q.stride), nullptr, nullptr, q.dtype, stream, sh.rot_interleaved ? 1 : 0), "qk_prepare");
+        return;
+    }
     if (k_pages.dtype != q.dtype || v_pages.dtype != q.dtype || !k_pages.contiguous() || !v_pages.contiguous() || k_pages.cols != nk ||
         v_pages.cols != nv || k_pages.rows != v_pages.rows)
         fail("qk_prepare: the pages must be contiguous [rows, %lld] and [rows, %lld] %s", (long long)nk, (long long)nv, dtype_name(q.dtype));
     if (positions == nullptr || slots == nullptr) fail("qk_prepare: positions and page rows are needed");
-    if (sh.norm_mode < 0 || sh.norm_mode > 2 || (sh.norm_mode != 0 && (sh.q_norm == nullptr || sh.k_norm == nullptr)))
+    if (sh.norm_mode < 0 || sh.norm_mode > 3 || ((sh.norm_mode == 1 || sh.norm_mode == 2) && (sh.q_norm == nullptr || sh.k_norm == nullptr)))
         fail("qk_prepare: norm mode %d needs its two weights", sh.norm_mode);
     if (sh.rot_dims < 0 || sh.rot_dims % 2 != 0 || sh.rot_dims > sh.dim || (sh.rot_dims > 0 && !(sh.rot_base > 0)))
         fail("qk_prepare: %d turned columns of %d (even, at most the head) and a positive base are needed", sh.rot_dims, sh.dim);
     check(mllm_qk_prepare(static_cast<const float*>(proj.data), i32(proj.stride), q_col, k_col, v_col, i32(proj.rows), sh.n_heads, sh.n_kv_heads,
                           sh.dim, sh.value_dim, sh.norm_mode, sh.q_norm, sh.k_norm, sh.eps, sh.rot_dims, sh.rot_base, positions, slots, q.data,
-                          i32(q.stride), k_pages.data, v_pages.data, q.dtype, stream), "qk_prepare");
+                          i32(q.stride), k_pages.data, v_pages.data, q.dtype, stream, sh.rot_interleaved ? 1 : 0), "qk_prepare");
 }
 
 void scored_attention(const Tensor2& q, const Tensor2& k_pages, const Tensor2& v_pages, const ScoredStep& step,
@@ -156,13 +167,15 @@ void scored_attention(const Tensor2& q, const Tensor2& k_pages, const Tensor2& v
     // (sigmoid weights and a gate per head: the matrix-core tiles and the split-key kernel in bfloat16 at their head
     // sizes; 32-bit and other sizes stay with the kernel below)
     const bool special = sh.sigmoid_weights || sh.gate_per_head;
+    const bool rows_only = sh.slope != nullptr || sh.sink != nullptr || sh.keep_first > 0;
     const bool special_ok = q.dtype == BF16 && (sh.dim == 32 || sh.dim == 64 || sh.dim == 128) && step.page_size >= sh.dim / 16 &&
                             (step.page_size & (step.page_size - 1)) == 0 && step.max_blocks <= 2048;
-    if (tuning().scored_shared_kernels && (!special || special_ok) && sh.dim == sh.value_dim && sh.dim % 8 == 0 && sh.dim <= 256 && (q.stride * q.esz()) % 16 == 0 && (sh.dim * q.esz()) % 16 == 0 &&
+    if (tuning().scored_shared_kernels && !rows_only && (!special || special_ok) && sh.dim == sh.value_dim && sh.dim % 8 == 0 && sh.dim <= 256 && (q.stride * q.esz()) % 16 == 0 && (sh.dim * q.esz()) % 16 == 0 &&
         (reinterpret_cast<uintptr_t>(q.data) & 15) == 0 && (g == nullptr || sh.gate_per_head || (ldg % 4 == 0 && (reinterpret_cast<uintptr_t>(g) & 15) == 0)) &&
         (reinterpret_cast<uintptr_t>(out.data) & 15) == 0 && (out.stride * out.esz()) % 8 == 0 &&
         step.cu_q != nullptr && step.ctx_len != nullptr && step.n_seqs > 0) {
-        const MllmScoreShape shape{sh.softcap, sh.chunk, sh.r1, sh.r2, sh.sigmoid_weights ? 1 : 0, sh.score_bias, sh.gate_per_head ? 1 : 0};
+        const MllmScoreShape shape{sh.softcap, sh.chunk, sh.r1, sh.r2, sh.sigmoid_weights ? 1 : 0, sh.score_bias, sh.gate_per_head ? 1 : 0,
+                                   sh.slope, sh.sink, sh.keep_first};
         AttentionArgs a;
         a.q = q; a.q_col = 0; a.n_heads = sh.n_heads; a.n_kv_heads = sh.n_kv_heads; a.head_dim = sh.dim;
         a.k_pages = k_pages; a.v_pages = v_pages; a.page_size = step.page_size;
@@ -176,7 +189,7 @@ void scored_attention(const Tensor2& q, const Tensor2& k_pages, const Tensor2& v
     check(mllm_scored_attention_rows(q.data, i32(q.stride), k_pages.data, v_pages.data, step.block_tables, step.max_blocks, step.token_seq,
                                      step.positions, i32(q.rows), sh.n_heads, sh.n_kv_heads, sh.dim, sh.value_dim, step.page_size, sh.scale,
                                      sh.softcap, sh.window, sh.chunk, sh.r1, sh.r2, g, ldg, out.data, i32(out.stride), q.dtype, stream,
-                                     sh.sigmoid_weights ? 1 : 0, sh.score_bias, sh.gate_per_head ? 1 : 0),
+                                     sh.sigmoid_weights ? 1 : 0, sh.score_bias, sh.gate_per_head ? 1 : 0, sh.slope, sh.sink, sh.keep_first),
           "scored_attention");
 }
 
@@ -301,6 +314,19 @@ void moe_act(const Tensor2& up, const Tensor2& logits, int ff, int top, float sc
     }
     check(mllm_moe_act(up.data, i32(up.stride), static_cast<const float*>(logits.data), i32(logits.stride), E, ff, i32(up.cols) - E * ff, top, scale,
                        out.data, i32(out.stride), wp, ldw, i32(up.rows), up.dtype, stream), "moe_act");
+}
+
+void moe_glu_act(const Tensor2& up, const Tensor2& logits, const MoeGlu& m, const Tensor2& out, hipStream_t stream) {
+    need_act(up, "moe_glu_act: up");
+    need_f32(logits, "moe_glu_act: the router's logits");
+    const int64_t n = static_cast<int64_t>(m.experts) * m.ff + m.shared_ff;
+    if (m.experts < 1 || m.ff < 1 || m.shared_ff < 0 || m.top < 1 || m.top > m.experts) fail("moe_glu_act: %d of %d experts of %d do not fit", m.top, m.experts, m.ff);
+    if (out.dtype != up.dtype || out.rows != up.rows || out.cols != n || up.cols != 2 * n) fail("moe_glu_act: up must be [T, %lld] and out [T, %lld], of one dtype", (long long)(2 * n), (long long)n);
+    if (logits.rows != up.rows || logits.cols != m.experts + (m.shared_gate ? 1 : 0)) fail("moe_glu_act: the logits must be [T, %d]", m.experts + (m.shared_gate ? 1 : 0));
+    if (out.data == up.data) fail("moe_glu_act: out must not be up");
+    check(mllm_moe_glu_act(up.data, i32(up.stride), static_cast<const float*>(logits.data), i32(logits.stride), m.experts, m.ff, m.shared_ff, m.top,
+                           m.scale, m.sigmoid_router ? 1 : 0, m.limit, m.shared_limit, m.alpha, m.weight_on_input ? 1 : 0, m.shared_gate ? 1 : 0,
+                           out.data, i32(out.stride), i32(up.rows), up.dtype, stream), "moe_glu_act");
 }
 
 void concat_cast(const Tensor2& a, const Tensor2& b, const Tensor2& out, hipStream_t stream) {

@@ -590,7 +590,10 @@ std::vector<CacheNeed> DecoderModel::cache_needs() const {
             mine.value_dim != theirs.value_dim || mine.state_bytes != theirs.state_bytes)
             fail("layer %d reads cache %d, which another kind of mixer writes", c.layer, c.cache);
         // the pages are kept for the widest window among the calls that read them (0: every key)
-        if ((theirs.kind & 1) && theirs.window > 0) needs[c.cache].window = mine.window > 0 ? std::max(theirs.window, mine.window) : 0;
+        if ((theirs.kind & 1) && theirs.window > 0) {
+            needs[c.cache].window = mine.window > 0 ? std::max(theirs.window, mine.window) : 0;
+            needs[c.cache].keep_first = std::max(theirs.keep_first, mine.keep_first);
+        }
     }
     return needs;
 }

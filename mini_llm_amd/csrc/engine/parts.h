@@ -118,6 +118,7 @@ struct CacheView {
 struct CacheNeed {
     int kind = 0;                        // bits: 1 keys and values in pages, 2 fixed-size state (3: both), 0 none
     int n_kv_heads = 0, head_dim = 0, window = 0;
+    int keep_first = 0;                  // with a window: the sequence's first keep_first positions are read for good
     int value_dim = -1;                  // width of a head's value rows; -1: as the keys; 0: the pages hold key rows only
     size_t state_bytes = 0;
 };

@@ -1,5 +1,5 @@
-// RMS norm, the block arrangements with a norm on both sides of each sub-layer and with a norm behind it only, and
-// the clamped gated feed-forward.
+// RMS norm, the block arrangements with a norm on both sides of each sub-layer, with a norm behind it only, and with
+// mixer and feed-forward side by side on one stream, and the clamped gated feed-forward.
 #include <algorithm>
 
 #include "parts.h"
@@ -273,6 +273,59 @@ private:
     int dtype_ = BF16, size_ = 0;     // size: the stream's width
 };
 
+// Mixer and feed-forward side by side, each behind a norm of its own, both reading the SAME stream:
+//   x += mixer(norm1(x)) + ff(norm2(x))
+// The feed-forward's input is normed before the mixer adds its result into the stream; then both add theirs. Norms:
+// [norm1] or [norm1, norm2].
+class ParallelNormBlock final : public Block {
+public:
+    ParallelNormBlock(std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f, std::vector<std::unique_ptr<Norm>> norms, const Params&)
+        : mixer_(std::move(m)), ff_(std::move(f)) {
+        if (!mixer_) fail("a parallel block needs a mixer");
+        if (norms.size() != (ff_ ? 2u : 1u)) fail("a parallel block has one norm per sub-layer (%d here), got %zu", ff_ ? 2 : 1, norms.size());
+        for (auto& n : norms) if (!n) fail("a parallel block was handed a missing norm");
+        norm1_ = std::move(norms[0]);
+        if (ff_) norm2_ = std::move(norms[1]);
+    }
+    void forward(const Tensor2& x, const StepView& step, const CacheView& cache, bool write, Arena& arena,
+                 hipStream_t s) const override {
+        const size_t outer = arena.mark();
+        Tensor2 h2;
+        if (ff_) h2 = norm2_->forward(x, nullptr, static_cast<int>(x.rows), arena, s);      // (before the mixer changes x)
+        const size_t mark = arena.mark();
+        {
+            NormedInput h(*norm1_, x);
+            mixer_->forward(h, step, cache, x, write, arena, s);
+        }
+        arena.release(mark);
+        if (ff_) {
+            NormedInput h(h2);
+            ff_->forward(h, step, x, arena, s);
+        }
+        arena.release(outer);
+    }
+    size_t workspace_bytes(int tokens) const override {
+        size_t a = mixer_->workspace_bytes(tokens) + 2 * norm1_->workspace_bytes(tokens);
+        if (ff_) a = std::max(a, ff_->workspace_bytes(tokens)) + 2 * norm2_->workspace_bytes(tokens);
+        return a + 1024;
+    }
+    CacheNeed cache_need() const override { return mixer_->cache_need(); }
+    void reserve(int max_seqs, hipStream_t s) const override {
+        mixer_->reserve(max_seqs, s);
+        if (ff_) ff_->reserve(max_seqs, s);
+    }
+    void add_cost(StepCost& c) const override {
+        norm1_->add_cost(c);
+        mixer_->add_cost(c);
+        if (ff_) { norm2_->add_cost(c); ff_->add_cost(c); }
+    }
+
+private:
+    std::unique_ptr<Mixer> mixer_;
+    std::unique_ptr<FeedForward> ff_;
+    std::unique_ptr<Norm> norm1_, norm2_;
+};
+
 // y = W_down( g sigmoid(alpha g) (u + 1) ) with g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit),
 // added into the stream it is handed. Parameters: limit, alpha, dtype; tensors gate.weight, up.weight,
 // down.weight ([out, in]).
@@ -327,6 +380,10 @@ void register_gated_parts() {
     register_block("sandwich_norm", [](std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f, std::vector<std::unique_ptr<Norm>> n,
                                        const Params& p) {
         return std::unique_ptr<Block>(new SandwichNormBlock(std::move(m), std::move(f), std::move(n), p));
+    });
+    register_block("parallel_norm", [](std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f, std::vector<std::unique_ptr<Norm>> n,
+                                       const Params& p) {
+        return std::unique_ptr<Block>(new ParallelNormBlock(std::move(m), std::move(f), std::move(n), p));
     });
     register_block("post_norm", [](std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f, std::vector<std::unique_ptr<Norm>> n,
                                    const Params& p) {

@@ -182,7 +182,7 @@ private:
 };
 
 // x += W_down(act(W_gate h + b_gate) * (W_up h + b_up)) + b_down. Gate and up are one joined product, rows
-// [gate: ff | up: ff]. Parameters: dtype, string activation (gelu_tanh); tensors gate_up.weight, gate_up.bias
+// [gate: ff | up: ff]. Parameters: dtype, string activation (gelu_tanh, silu); tensors gate_up.weight, gate_up.bias
 // (optional), down.weight, down.bias (optional).
 class GatedMLP final : public FeedForward {
 public:
@@ -190,7 +190,8 @@ public:
         dtype_ = p.integer("dtype");
         const std::string& act = p.string("activation");
         if (act == "gelu_tanh") act_ = GELU_TANH;
-        else fail("gated_mlp: unknown activation '%s' (known: gelu_tanh)", act.c_str());
+        else if (act == "silu") act_ = GLU_SILU;
+        else fail("gated_mlp: unknown activation '%s' (known: gelu_tanh, silu)", act.c_str());
         gate_up_ = Linear(p.weights("gate_up.weight"), p.weights_or_null("gate_up.bias"));
         down_ = Linear(p.weights("down.weight"), p.weights_or_null("down.bias"));
         if (gate_up_.out_features() != 2 * down_.in_features()) fail("gated_mlp: the products' shapes do not fit");

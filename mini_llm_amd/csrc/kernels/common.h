@@ -238,7 +238,8 @@ __device__ __forceinline__ void epilogue(int mode, float acc, float bias, void* 
 
 #include "score_shape.h"
 
-// A score (already times its scale, natural units) of query head with bias numbers r1, r2 at distance `dist`.
+// A score (already times its scale, natural units) of query head with bias numbers r1, r2 at distance `dist`
+// (with a linear distance bias instead of the logarithmic one, r1 is the head's slope: mllm_bias_r1).
 // FAST (the bfloat16 kernels): tanh through one hardware exponential and a reciprocal, the logarithm by the hardware
 // instruction (at distance 0 its argument is exactly 1); otherwise the library's full-precision functions.
 template <bool FAST = false>
@@ -250,8 +251,14 @@ __device__ __forceinline__ float mllm_shaped_score(float s, const MllmScoreShape
     if (sh.r1 != nullptr) {
         const float a = r2 * static_cast<float>(dist);
         s -= r1 * (FAST ? __logf(1.f + a) : log1pf(a));
+    } else if (sh.slope != nullptr) {
+        s -= r1 * static_cast<float>(dist);          // (the caller hands the head's slope over as r1)
     }
     return s;
+}
+// The first bias number of head h: r1[h], or the linear bias's slope[h], or 0.
+__device__ __forceinline__ float mllm_bias_r1(const MllmScoreShape& sh, int h) {
+    return sh.r1 != nullptr ? sh.r1[h] : (sh.slope != nullptr ? sh.slope[h] : 0.f);
 }
 #define MLLM_LOG2E 1.44269504088896340736f
 

@@ -194,14 +194,15 @@ __global__ void concat_cast_kernel(const float* __restrict__ a, const float* __r
 }
 
 // out[t, j] = act(gu[t, j]) * gu[t, F + j]: the two halves of a joined gate/up product
-template <typename T>
+template <typename T, bool SILU>
 __global__ void glu_act_kernel(const T* __restrict__ gu, int ld, int F, T* __restrict__ out, int ldo, long long total) {
     const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= total) return;
     const long long t = i / F;
     const int j = static_cast<int>(i % F);
     const float g = to_float(gu[t * ld + j]), u = to_float(gu[t * ld + F + j]);
-    out[t * ldo + j] = from_float<T>((sizeof(T) == 4 ? gelu_tanh_precise(g) : gelu_tanh(g)) * u);
+    if (SILU) out[t * ldo + j] = from_float<T>(g / (1.f + (sizeof(T) == 4 ? expf(-g) : __expf(-g))) * u);
+    else out[t * ldo + j] = from_float<T>((sizeof(T) == 4 ? gelu_tanh_precise(g) : gelu_tanh(g)) * u);
 }
 
 
@@ -352,14 +353,16 @@ int mllm_concat_cast(const float* a, const float* b, int T, int D, void* out, in
     return 0;
 }
 
-// -1: an activation other than the tanh form of GELU (code 1)
+// -1: an activation other than the tanh form of GELU (code 1) or silu (code 5)
 int mllm_glu_act(const void* gu, int ld, int T, int F, int act, void* out, int ldo, int dtype, hipStream_t stream) {
     if (T <= 0 || F <= 0) return 0;
-    if (act != EPI_GELU_TANH) return -1;
+    if (act != EPI_GELU_TANH && act != 5) return -1;
     const long long total = static_cast<long long>(T) * F;
     const int blocks = static_cast<int>((total + 255) / 256);
-    if (dtype == MLLM_F32) glu_act_kernel<float><<<blocks, 256, 0, stream>>>(static_cast<const float*>(gu), ld, F, static_cast<float*>(out), ldo, total);
-    else glu_act_kernel<bf16_t><<<blocks, 256, 0, stream>>>(static_cast<const bf16_t*>(gu), ld, F, static_cast<bf16_t*>(out), ldo, total);
+#define GLU_ACT(TYPE, SILU) glu_act_kernel<TYPE, SILU><<<blocks, 256, 0, stream>>>(static_cast<const TYPE*>(gu), ld, F, static_cast<TYPE*>(out), ldo, total)
+    if (dtype == MLLM_F32) { if (act == 5) GLU_ACT(float, true); else GLU_ACT(float, false); }
+    else { if (act == 5) GLU_ACT(bf16_t, true); else GLU_ACT(bf16_t, false); }
+#undef GLU_ACT
     MLLM_LAUNCH_CHECK();
     return 0;
 }

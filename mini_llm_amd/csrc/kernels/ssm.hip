@@ -16,6 +16,8 @@ __device__ __forceinline__ float softplus_precise(float v) { return fmaxf(v, 0.f
 
 // out[t, ch] = silu(bias[ch] + sum_j w[ch, j] * in(t - (taps - 1 - j), ch)): inputs before the portion come
 // from the slot's carried rows (zeros for a fresh request: the slot was cleared). One thread per (t, ch).
+// SILU false: the convolution alone, no activation; the bias may be null.
+template <bool SILU>
 __global__ void conv_silu_kernel(const float* __restrict__ proj, int ld, int col0, int C, const float* __restrict__ w,
                                  const float* __restrict__ bias, int taps, const int* __restrict__ token_seq,
                                  const int* __restrict__ cu_q, const int* __restrict__ state_slots,
@@ -28,7 +30,7 @@ __global__ void conv_silu_kernel(const float* __restrict__ proj, int ld, int col
     if (slot < 0) return;
     const int first = cu_q[b], k = t - first;
     float* carried = state + static_cast<size_t>(slot) * slot_floats;
-    float acc = bias[ch];
+    float acc = bias != nullptr ? bias[ch] : 0.f;
     for (int j = 0; j < taps; ++j) {
         const int idx = k - (taps - 1 - j);
         const float v = idx >= 0 ? proj[static_cast<size_t>(first + idx) * ld + col0 + ch]
@@ -38,7 +40,7 @@ __global__ void conv_silu_kernel(const float* __restrict__ proj, int ld, int col
         // carried rows move up by one behind the read, and the token's input becomes the newest
         if (carry && j >= 1) carried[static_cast<size_t>(j - 1) * C + ch] = v;
     }
-    out[static_cast<size_t>(t) * ldo + ch] = silu_precise(acc);
+    out[static_cast<size_t>(t) * ldo + ch] = SILU ? silu_precise(acc) : acc;
 }
 
 // out[t, ch] = in[t, ch] + sum_j w[ch, j] * in(t - (taps - 1 - j), ch): the convolution added onto its own input,
@@ -573,19 +575,24 @@ static int stream_conv_single_launch(float* x, int ldx, const float* y, int ldy,
 
 extern "C" {
 
-// Convolution + silu of columns [col0, col0 + C) of proj's rows into out [T, C]; then, with `write`, the
+// Convolution + silu (activation 0: the convolution alone, the bias may be null) of columns [col0, col0 + C) of
+// proj's rows into out [T, C]; then, with `write`, the
 // slots' carried rows are brought up to date (a second kernel: it overwrites what the first one reads).
 // -1: taps outside 1..16.
 int mllm_conv_silu(const float* proj, int ld, int col0, int C, const float* w, const float* bias, int taps,
                    const int* token_seq, const int* cu_q, const int* state_slots, float* state, size_t slot_floats,
-                   float* out, int ldo, int T, int B, int write, hipStream_t stream) {
+                   float* out, int ldo, int T, int B, int write, hipStream_t stream, int activation) {
     if (T <= 0 || C <= 0) return 0;
-    if (taps < 1 || taps > 16) return -1;
+    if (taps < 1 || taps > 16 || (activation != 0 && bias == nullptr)) return -1;
     const long long total = static_cast<long long>(T) * C;
     // (one token a sequence: the convolution's kernel brings the carried rows up to date itself)
     const bool single = T == B && write && taps > 1;
-    conv_silu_kernel<<<static_cast<int>((total + 255) / 256), 256, 0, stream>>>(proj, ld, col0, C, w, bias, taps, token_seq, cu_q,
-                                                                                state_slots, state, slot_floats, out, ldo, total, single ? 1 : 0);
+    if (activation != 0)
+        conv_silu_kernel<true><<<static_cast<int>((total + 255) / 256), 256, 0, stream>>>(proj, ld, col0, C, w, bias, taps, token_seq, cu_q,
+                                                                                          state_slots, state, slot_floats, out, ldo, total, single ? 1 : 0);
+    else
+        conv_silu_kernel<false><<<static_cast<int>((total + 255) / 256), 256, 0, stream>>>(proj, ld, col0, C, w, bias, taps, token_seq, cu_q,
+                                                                                           state_slots, state, slot_floats, out, ldo, total, single ? 1 : 0);
     MLLM_LAUNCH_CHECK();
     if (write && taps > 1 && !single) {
         const long long pairs = static_cast<long long>(B) * C;

@@ -115,7 +115,9 @@ int CacheManager::commit(int64_t id, int new_len) {
         int keep_from = first_key / gs.page_size;
         auto& tab = rc.tables[g];
         int upto = std::min(keep_from, static_cast<int>(tab.size()));
-        for (int b = rc.first_live[g]; b < upto; ++b) {
+        // (the pages of the kept first keys stay with the request until it ends)
+        const int kept = gs.keep_first > 0 ? (gs.keep_first + gs.page_size - 1) / gs.page_size : 0;
+        for (int b = std::max(rc.first_live[g], kept); b < upto; ++b) {
             if (tab[b] >= 0) {
                 pools_[g].give_back(tab[b]);
                 tab[b] = -1;

@@ -21,6 +21,7 @@ struct GroupSpec {
     int page_size = 16;   // tokens per page
     int n_pages = 0;      // pages in this group's pool
     int window = 0;       // 0: every earlier key is kept; W>0: only the last W keys are needed
+    int keep_first = 0;   // with a window: the pages that hold the first keep_first keys are never given back early
 };
 
 class PagePool {
