@@ -30,6 +30,7 @@ def _rt():
     vp, i64, i = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
     sigs = {
         "mllm_cache_create": (vp, [i, _i32p, _i32p, _i32p, i]),
+        "mllm_cache_create_keeping": (vp, [i, _i32p, _i32p, _i32p, _i32p, i]),
         "mllm_cache_destroy": (None, [vp]),
         "mllm_cache_add_request": (i, [vp, i64]),
         "mllm_cache_has_request": (i, [vp, i64]),
@@ -83,6 +84,7 @@ class GroupSpec:
     page_size: int
     n_pages: int
     window: int = 0      # 0: all keys are kept; W > 0: only the last W keys are needed
+    keep_first: int = 0  # with a window: the pages of the first keep_first keys stay until the request ends
 
 
 class CacheManager:
@@ -96,7 +98,8 @@ class CacheManager:
         ps = (ctypes.c_int * max(n, 1))(*[g.page_size for g in self.groups])
         npg = (ctypes.c_int * max(n, 1))(*[g.n_pages for g in self.groups])
         win = (ctypes.c_int * max(n, 1))(*[g.window for g in self.groups])
-        self._h = self._lib.mllm_cache_create(n, ps, npg, win, self.n_state_slots)
+        keep = (ctypes.c_int * max(n, 1))(*[g.keep_first for g in self.groups])
+        self._h = self._lib.mllm_cache_create_keeping(n, ps, npg, win, keep, self.n_state_slots)
         if not self._h:
             raise ValueError(f"invalid cache groups {self.groups} or slots {n_state_slots}")
 

@@ -399,13 +399,15 @@ bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_
         check(mllm_scored_attention_rows(a.q.data, static_cast<int>(a.q.stride), a.k_pages.data, a.v_pages.data, a.block_tables, a.max_blocks,
                                          a.token_seq, a.positions, n_rows, a.n_heads, a.n_kv_heads, a.head_dim, a.head_dim, a.page_size,
                                          a.scale, a.shape->softcap, a.window, a.shape->chunk, a.shape->r1, a.shape->r2, a.gate, a.gate_stride,
-                                         a.out.data, static_cast<int>(a.out.stride), a.q.dtype, stream), "scored_attention (rows)");
+                                         a.out.data, static_cast<int>(a.out.stride), a.q.dtype, stream, a.shape->sigmoid, a.shape->score_bias,
+                                         a.shape->gate_per_head, a.shape->slope, a.shape->sink, a.shape->keep_first), "scored_attention (rows)");
     };
     if (a.shape != nullptr && a.q_col != 0) fail("paged_attention: shaped scores take queries from column 0");
-    if (a.shape != nullptr && (a.shape->sigmoid || a.shape->gate_per_head) &&
+    if (a.shape != nullptr && a.shape->keep_first > 0 && a.window <= 0) fail("paged_attention: kept first positions go with a window");
+    if (a.shape != nullptr && a.shape->sigmoid &&
         !(a.q.dtype == BF16 && (a.head_dim == 32 || a.head_dim == 64 || a.head_dim == 128) && pow2(a.page_size) && a.page_size >= a.head_dim / 16 &&
           a.max_blocks <= 2048 && (a.max_q_len == 1 || (a.cu_q != nullptr && a.ctx_len != nullptr))))
-        fail("paged_attention: sigmoid weights and a gate per head are taken in bfloat16 at head sizes 32, 64 and 128 only");
+        fail("paged_attention: sigmoid weights are taken in bfloat16 at head sizes 32, 64 and 128 only");
     const int lpk = a.head_dim * esz / 16;
     const bool single_ok = lpk >= 2 && pow2(lpk) && pow2(a.page_size) && a.max_blocks <= 4096;
     const bool decode = a.max_q_len == 1 && single_ok;
@@ -482,7 +484,8 @@ bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_
         bool merge_kernel = false;
         decode_launch_shape(pairs, a.max_ctx_len, unmerged, &nsplit, &waves, &merge_kernel);
         // (sigmoid weights have no sum to divide by afterwards: the kernel merges its own splits, however many)
-        if (a.shape != nullptr && a.shape->sigmoid) merge_kernel = false;
+        // (nor does the merge kernel know a gate of one value per head)
+        if (a.shape != nullptr && (a.shape->sigmoid || (a.gate != nullptr && a.shape->gate_per_head))) merge_kernel = false;
         unmerged = unmerged && nsplit > 1 && !merge_kernel;
         float* ws = decode_partials(nsplit > 1 ? static_cast<size_t>(pairs) * nsplit * (a.head_dim + 2) : 1, stream);
         int* counters = decode_counters(pairs, stream);

@@ -164,13 +164,12 @@ void scored_attention(const Tensor2& q, const Tensor2& k_pages, const Tensor2& v
     // keys and values of one width: the kernels that every attention of the engine runs on (tiles of queries for
     // prompt portions, split keys for single tokens), with the shaping handed on; they fall back by themselves to
     // the one-wavefront-per-row kernel below for sizes they do not take
-    // (sigmoid weights and a gate per head: the matrix-core tiles and the split-key kernel in bfloat16 at their head
-    // sizes; 32-bit and other sizes stay with the kernel below)
-    const bool special = sh.sigmoid_weights || sh.gate_per_head;
-    const bool rows_only = sh.slope != nullptr || sh.sink != nullptr || sh.keep_first > 0;
+    // (sigmoid weights: the matrix-core tiles and the split-key kernel in bfloat16 at their head sizes; 32-bit and
+    // other sizes stay with the kernel below)
+    const bool special = sh.sigmoid_weights;
     const bool special_ok = q.dtype == BF16 && (sh.dim == 32 || sh.dim == 64 || sh.dim == 128) && step.page_size >= sh.dim / 16 &&
                             (step.page_size & (step.page_size - 1)) == 0 && step.max_blocks <= 2048;
-    if (tuning().scored_shared_kernels && !rows_only && (!special || special_ok) && sh.dim == sh.value_dim && sh.dim % 8 == 0 && sh.dim <= 256 && (q.stride * q.esz()) % 16 == 0 && (sh.dim * q.esz()) % 16 == 0 &&
+    if (tuning().scored_shared_kernels && (!special || special_ok) && sh.dim == sh.value_dim && sh.dim % 8 == 0 && sh.dim <= 256 && (q.stride * q.esz()) % 16 == 0 && (sh.dim * q.esz()) % 16 == 0 &&
         (reinterpret_cast<uintptr_t>(q.data) & 15) == 0 && (g == nullptr || sh.gate_per_head || (ldg % 4 == 0 && (reinterpret_cast<uintptr_t>(g) & 15) == 0)) &&
         (reinterpret_cast<uintptr_t>(out.data) & 15) == 0 && (out.stride * out.esz()) % 8 == 0 &&
         step.cu_q != nullptr && step.ctx_len != nullptr && step.n_seqs > 0) {

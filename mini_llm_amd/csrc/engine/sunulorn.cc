@@ -260,12 +260,17 @@ void sunulorn_assemble(const Json& config, const std::map<std::string, Tensor2>&
         const LayerConfig& l = c.layers[i];
         const MixerConfig& x = l.mix;
         const std::string L = "l" + std::to_string(i) + ".", M = L + "mix.";
+        // Value heads narrower than the keys are made as wide: zero rows in the values' projection (and the gate's), zero
+        // columns in the output projection. The result is the same, and the attention kernels that every model shares
+        // (key tiles on the matrix cores, split keys) take keys and values of one width only.
+        const int64_t e = (x.vdim < x.dim && x.dim % 16 == 0) ? x.dim : x.vdim;
+        auto widened_rows = [&](const Tensor2& w) { return e == x.vdim ? w : out.store.pad_row_blocks(w, x.vdim, e); };
         Params p;
         p.num["heads"] = static_cast<double>(x.heads); p.num["kv_heads"] = static_cast<double>(x.kv_heads);
-        p.num["dim"] = static_cast<double>(x.dim); p.num["value_dim"] = static_cast<double>(x.vdim);
+        p.num["dim"] = static_cast<double>(x.dim); p.num["value_dim"] = static_cast<double>(e);
         p.num["scale"] = x.scale; p.num["eps"] = c.eps; p.num["dtype"] = dtype;
         p.str["qk_norm"] = "none";
-        p.tensor["out.weight"] = t.at(M + "o");
+        p.tensor["out.weight"] = e == x.vdim ? t.at(M + "o") : out.store.pad_col_blocks(t.at(M + "o"), x.vdim, e);
         if (x.kind == MixerConfig::ConvAttention) {
             p.num["values_from_keys"] = 1;
             p.num["rot_dims"] = static_cast<double>(x.rot_dims); p.num["rot_base"] = x.rot_base; p.num["rot_interleaved"] = 1;
@@ -278,9 +283,9 @@ void sunulorn_assemble(const Json& config, const std::map<std::string, Tensor2>&
             p.str["qk_norm"] = "unit_after";
             p.num["window"] = static_cast<double>(x.window); p.num["keep_first"] = static_cast<double>(x.window > 0 ? x.keep_first : 0);
             p.num["gated"] = 1;
-            p.tensor["in.weight"] = out.store.join_rows({t.at(M + "q"), t.at(M + "k"), t.at(M + "v"), t.at(M + "g")});
+            p.tensor["in.weight"] = out.store.join_rows({t.at(M + "q"), t.at(M + "k"), widened_rows(t.at(M + "v")), widened_rows(t.at(M + "g"))});
             // (the gate's projection has no bias)
-            p.tensor["in.bias"] = out.store.join_rows({column(t.at(M + "q.b")), column(t.at(M + "k.b")), column(t.at(M + "v.b")), column(out.store.zeros(x.heads * x.vdim))});
+            p.tensor["in.bias"] = out.store.join_rows({column(t.at(M + "q.b")), column(t.at(M + "k.b")), widened_rows(column(t.at(M + "v.b"))), column(out.store.zeros(x.heads * e))});
             p.tensor["out.bias"] = t.at(M + "o.b");
         } else {
             p.num["gated"] = 1; p.num["gate_per_head"] = 1;
@@ -293,8 +298,8 @@ void sunulorn_assemble(const Json& config, const std::map<std::string, Tensor2>&
                 p.tensor["in.weight"] = out.store.join_rows({t.at(M + "q"), t.at(M + "g")});
                 p.tensor["in.bias"] = out.store.join_rows({column(t.at(M + "q.b")), column(out.store.zeros(x.heads))});
             } else {
-                p.tensor["in.weight"] = out.store.join_rows({t.at(M + "q"), t.at(M + "k"), t.at(M + "v"), t.at(M + "g")});
-                p.tensor["in.bias"] = out.store.join_rows({column(t.at(M + "q.b")), column(t.at(M + "k.b")), column(t.at(M + "v.b")), column(out.store.zeros(x.heads))});
+                p.tensor["in.weight"] = out.store.join_rows({t.at(M + "q"), t.at(M + "k"), widened_rows(t.at(M + "v")), t.at(M + "g")});
+                p.tensor["in.bias"] = out.store.join_rows({column(t.at(M + "q.b")), column(t.at(M + "k.b")), widened_rows(column(t.at(M + "v.b"))), column(out.store.zeros(x.heads))});
             }
         }
         std::unique_ptr<Mixer> mixer = build_mixer("scored_attention", p);

@@ -323,6 +323,30 @@ Tensor2 DeviceTensors::join_cols(const std::vector<Tensor2>& parts) {
     return Tensor2(base, parts[0].dtype, parts[0].rows, cols);
 }
 
+Tensor2 DeviceTensors::pad_row_blocks(const Tensor2& t, int64_t block, int64_t padded) {
+    if (block < 1 || padded < block || t.rows % block != 0 || !t.contiguous()) throw WeightsError("pad_row_blocks: contiguous rows in whole blocks are needed");
+    const int64_t n = t.rows / block;
+    const size_t row_bytes = static_cast<size_t>(t.cols) * t.esz();
+    char* base = static_cast<char*>(allocate(static_cast<size_t>(n * padded) * row_bytes, true));
+    for (int64_t b = 0; b < n; ++b)
+        if (row_bytes > 0 && hipMemcpy(base + static_cast<size_t>(b * padded) * row_bytes, static_cast<const char*>(t.data) + static_cast<size_t>(b * block) * row_bytes,
+                                       static_cast<size_t>(block) * row_bytes, hipMemcpyDeviceToDevice) != hipSuccess)
+            throw WeightsError("pad_row_blocks: the copy on the device failed");
+    return Tensor2(base, t.dtype, n * padded, t.cols);
+}
+
+Tensor2 DeviceTensors::pad_col_blocks(const Tensor2& t, int64_t block, int64_t padded) {
+    if (block < 1 || padded < block || t.cols % block != 0 || !t.contiguous()) throw WeightsError("pad_col_blocks: contiguous columns in whole blocks are needed");
+    const int64_t n = t.cols / block;
+    const size_t esz = t.esz(), src_pitch = static_cast<size_t>(t.cols) * esz, dst_pitch = static_cast<size_t>(n * padded) * esz;
+    char* base = static_cast<char*>(allocate(static_cast<size_t>(t.rows) * dst_pitch, true));
+    for (int64_t b = 0; b < n; ++b)
+        if (t.rows > 0 && hipMemcpy2D(base + static_cast<size_t>(b * padded) * esz, dst_pitch, static_cast<const char*>(t.data) + static_cast<size_t>(b * block) * esz, src_pitch,
+                                      static_cast<size_t>(block) * esz, static_cast<size_t>(t.rows), hipMemcpyDeviceToDevice) != hipSuccess)
+            throw WeightsError("pad_col_blocks: the copy on the device failed");
+    return Tensor2(base, t.dtype, t.rows, n * padded);
+}
+
 Tensor2 DeviceTensors::zeros(int64_t n) {
     if (n < 0) throw WeightsError("zeros: a negative size");
     return Tensor2(allocate(static_cast<size_t>(n) * 4, true), F32, 1, n);

@@ -158,6 +158,11 @@ public:
     Tensor2 join_cols(const std::vector<Tensor2>& parts);
     // n zeros ([1, n] fp32).
     Tensor2 zeros(int64_t n);
+    // Every block of `block` consecutive rows followed by zero rows up to `padded` rows a block ([rows / block * padded,
+    // cols], a copy on the device); pad_col_blocks: the same over the columns. A head's narrower rows or columns made
+    // as wide as another's, the added ones zero.
+    Tensor2 pad_row_blocks(const Tensor2& t, int64_t block, int64_t padded);
+    Tensor2 pad_col_blocks(const Tensor2& t, int64_t block, int64_t padded);
     size_t bytes() const { return bytes_; }
 
 private:

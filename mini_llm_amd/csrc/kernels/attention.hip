@@ -175,7 +175,13 @@ paged_attention_tiled(const T* __restrict__ q, int q_stride, int q_col, const T*
     int k_lo = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
     int my_lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     if (SHAPED && shape.chunk > 0) { k_lo = p_first - p_first % shape.chunk; my_lo = p - p % shape.chunk; }
-    const float r1 = (SHAPED && shape.r1) ? shape.r1[blockIdx.x] : 0.f, r2 = (SHAPED && shape.r1) ? shape.r2[blockIdx.x] : 0.f;
+    const float r1 = SHAPED ? mllm_bias_r1(shape, blockIdx.x) : 0.f, r2 = (SHAPED && shape.r1) ? shape.r2[blockIdx.x] : 0.f;
+    // A window may keep the sequence's first kf positions visible: key tiles that lie wholly in front of the window's
+    // first tile and hold kept keys run first (n_head of them); tile number vt is key tile tile_of(vt).
+    const int kf = (SHAPED && window > 0) ? shape.keep_first : 0;
+    const int kt_first = k_lo / TL_BK, kt_last = p_last / TL_BK;
+    const int n_head = kf > 0 ? min((kf + TL_BK - 1) / TL_BK, kt_first) : 0;
+    const int vt_last = n_head + kt_last - kt_first;
     // the last position any of this wavefront's queries may see (uniform over the wavefront)
     const int wave_last = start + min(q0 + wave * 16 + 15, q_len - 1);
     const int* table = block_tables + static_cast<size_t>(b) * max_blocks;
@@ -193,13 +199,14 @@ paged_attention_tiled(const T* __restrict__ q, int q_stride, int q_col, const T*
     }
     float m = -INFINITY, l = 0.f;
 
-    for (int k0 = k_lo - k_lo % TL_BK; k0 <= p_last; k0 += TL_BK) {
+    for (int vt = 0; vt <= vt_last; ++vt) {
+        const int k0 = (vt < n_head ? vt : vt - n_head + kt_first) * TL_BK;
         __syncthreads();                           // the previous tile's readers are done
         // stage 64 keys and values: thread t has key t % 64 and a quarter of its dims. Keys outside
         // [k_lo, p_last] are not in the pages (not written yet, or given back by a window): zeros.
         {
             const int key = tid % TL_BK, part = tid / TL_BK, j = k0 + key;
-            const bool live = j >= k_lo && j <= p_last;
+            const bool live = (j >= k_lo || j < kf) && j <= p_last;
             size_t row = 0;
             if (live) row = static_cast<size_t>(table[j / page_size]) * page_size + j % page_size;
             const T* kp = k_pages + row * kv_dim + kv_off;
@@ -238,7 +245,7 @@ paged_attention_tiled(const T* __restrict__ q, int q_stride, int q_col, const T*
             for (int i = 0; i < 4; ++i) {
                 const int j = k0 + 16 * g + 4 * G + i;
                 if (SHAPED) s[g][i] = mllm_shaped_score<sizeof(T) == 2>(s[g][i], shape, r1, r2, max(p - j, 0)) * MLLM_LOG2E;
-                s[g][i] = (j <= p && j >= my_lo) ? s[g][i] : -INFINITY;
+                s[g][i] = (j <= p && (j >= my_lo || j < kf)) ? s[g][i] : -INFINITY;
                 mx = fmaxf(mx, s[g][i]);
             }
         const float m_new = fmaxf(m, rows_max(mx));
@@ -269,14 +276,26 @@ paged_attention_tiled(const T* __restrict__ q, int q_stride, int q_col, const T*
         }
     }
     if (!q_ok) return;
+    if (SHAPED && shape.sink != nullptr) {
+        // the sink: one more term of the denominator, exp(sink), without a value (the maximum is in base 2)
+        const float sk = shape.sink[blockIdx.x] * MLLM_LOG2E, m_new = fmaxf(m, sk);
+        const float a = (m == -INFINITY) ? 0.f : exp2_for<T>(m - m_new);
+        l = l * a + exp2_for<T>(sk - m_new);
+#pragma unroll
+        for (int c = 0; c < DC; ++c) o[c] *= a;
+    }
     // lane holds O^T[dims 16c + 4G + i][its query]
     const float inv_l = 1.f / l;
+    const bool head_gate = SHAPED && gate != nullptr && shape.gate_per_head;
+    const float hg = head_gate ? 1.f / (1.f + expf(-gate[static_cast<size_t>(q_begin + qi) * ldg + h])) : 1.f;
     T* op = out + static_cast<size_t>(q_begin + qi) * out_stride + h * head_dim + 4 * G;
 #pragma unroll
     for (int c = 0; c < DC; ++c) {
         if (c < n_c) {
             f32x4_t r = o[c] * inv_l;
-            if (SHAPED && gate != nullptr) {
+            if (head_gate) {
+                r *= hg;
+            } else if (SHAPED && gate != nullptr) {
                 const float* gp = gate + static_cast<size_t>(q_begin + qi) * ldg + h * head_dim + 4 * G + 16 * c;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) r[i] *= 1.f / (1.f + expf(-gp[i]));

@@ -108,25 +108,32 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
     const int p = positions[t];
     int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     if (SHAPED && shape.chunk > 0) lo = p - p % shape.chunk;
-    const float r1 = (SHAPED && shape.r1) ? shape.r1[h] : 0.f, r2 = (SHAPED && shape.r1) ? shape.r2[h] : 0.f;
+    const float r1 = SHAPED ? mllm_bias_r1(shape, h) : 0.f, r2 = (SHAPED && shape.r1) ? shape.r2[h] : 0.f;
     const float sbias = (SIGMOID && shape.score_bias) ? shape.score_bias[h] : 0.f;
-    const int n_keys = p - lo + 1;
+    // The visible keys are counted through: first the kept first positions that lie in front of the window (none
+    // without them), then the window's. Key number v stands at position key_at(v); kb, ke and the loops below count
+    // in these numbers, so the splits share kept and window keys alike.
+    const int kf = (SHAPED && window > 0 && shape.keep_first > 0) ? min(shape.keep_first, lo) : 0;
+    const int shift_pos = lo - kf;
+    auto key_at = [&](int v) { return v < kf ? v : v + shift_pos; };
+    const int n_keys = p - lo + 1 + kf;
     const int per = (n_keys + nsplit - 1) / nsplit;
-    const int kb = lo + split * per;
-    const int ke = min(p + 1, kb + per);
+    const int kb = split * per;
+    const int ke = min(n_keys, kb + per);
     // With `slots`, the token's own key and value are not in the pages yet: they are read from
     // its row of q (columns k_col, v_col), and written to the pages by the first query head of
     // each key/value head. That key is taken by one lane group after the loop over the pages.
     const bool append = slots != nullptr;
-    const bool own_here = append && ke == p + 1 && kb <= p;     // this workgroup's range holds the token itself
-    const int ke_pages = own_here ? p : ke;                     // keys [kb, ke_pages) come from the pages
+    const bool own_here = append && ke == n_keys && kb <= n_keys - 1;     // this workgroup's range holds the token itself
+    const int ke_pages = own_here ? n_keys - 1 : ke;                      // keys [kb, ke_pages) come from the pages
     const size_t col = static_cast<size_t>(hk) * DH + c * EPL;
     const int shift = __ffs(page_size) - 1;                     // page sizes are powers of two
 
     // The block table entries of this workgroup's keys go to LDS first, so that no key load waits
     // for a table load.
-    const int first_blk = whole_row ? 0 : kb >> shift;
-    const int n_blk = ke_pages > kb ? ((ke_pages - 1) >> shift) - first_blk + 1 : 0;
+    // (with kept first positions the keys of a range need not be neighbours: the table from block 0 on)
+    const int first_blk = (whole_row || kf > 0) ? 0 : key_at(kb) >> shift;
+    const int n_blk = ke_pages > kb ? (key_at(ke_pages - 1) >> shift) - first_blk + 1 : 0;
     if (!whole_row) {
         const int* gtable = gtable_row + first_blk;
         for (int i = threadIdx.x; i < n_blk; i += blockDim.x) sm_table[i] = gtable[i];
@@ -158,6 +165,9 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
     float m = M0, l = 0.f, o[EPL];
 #pragma unroll
     for (int e = 0; e < EPL; ++e) o[e] = 0.f;
+    // A sink is one more term of the denominator, exp(sink), without a value: one lane group of the first split
+    // starts from it instead of from nothing.
+    if (SHAPED && !SIGMOID && shape.sink != nullptr && split == 0 && wave == 0 && g == 0) { m = shape.sink[h] * MLLM_LOG2E; l = 1.f; }
 
     // A wavefront takes UNR groups of 64/LPK keys at a time. All their loads are issued
     // first, unconditionally (a key beyond the range loads the last key of the range again and is
@@ -169,7 +179,7 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
         uint4 kraw[UNR], vraw[UNR];
 #pragma unroll
         for (int u = 0; u < UNR; ++u) {
-            const int j = min(j0 + u * group_keys + g, ke_pages - 1);
+            const int j = key_at(min(j0 + u * group_keys + g, ke_pages - 1));
             const size_t row = (static_cast<size_t>(sm_table[(j >> shift) - first_blk]) << shift) + (j & mask);
             kraw[u] = load_stream16(k_pages + row * kv_dim + col);
             vraw[u] = load_stream16(v_pages + row * kv_dim + col);
@@ -185,7 +195,7 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
             for (int e = 0; e < EPL; ++e) d = fmaf(qf[e], kf[e], d);
             d = group_sum<LPK>(d);
             const bool valid = j0 + u * group_keys + g < ke_pages;
-            if (SHAPED) d = mllm_shaped_score<sizeof(T) == 2>(d, shape, r1, r2, valid ? p - (j0 + u * group_keys + g) : 0) * MLLM_LOG2E;
+            if (SHAPED) d = mllm_shaped_score<sizeof(T) == 2>(d, shape, r1, r2, valid ? p - key_at(j0 + u * group_keys + g) : 0) * MLLM_LOG2E;
             if (SIGMOID) {
                 const float w = 1.f / (1.f + exp2_for<T>(-(d + sbias * MLLM_LOG2E)));
                 dot[u] = valid ? w : 0.f;             // the weight itself

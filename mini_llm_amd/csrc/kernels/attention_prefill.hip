@@ -96,8 +96,16 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
     int k_lo = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
     const int chunk = SHAPED ? shape.chunk : 0;
     if (chunk > 0) k_lo = p_first - p_first % chunk;
-    const float r1 = (SHAPED && shape.r1) ? shape.r1[blockIdx.x] : 0.f, r2 = (SHAPED && shape.r1) ? shape.r2[blockIdx.x] : 0.f;
+    const float r1 = SHAPED ? mllm_bias_r1(shape, blockIdx.x) : 0.f, r2 = (SHAPED && shape.r1) ? shape.r2[blockIdx.x] : 0.f;
     const float sbias = (SIGMOID && shape.score_bias) ? shape.score_bias[blockIdx.x] : 0.f;
+    // A window may keep the sequence's first kf positions visible. Key tiles that lie wholly in front of the window's
+    // first tile and hold kept keys run first (n_head of them); the tiles are counted through, tile number vt being
+    // key tile tile_of(vt). Their pages stay with the request, as the window's do.
+    const int kf = (SHAPED && window > 0) ? shape.keep_first : 0;
+    const int kt_first = k_lo / PF_BN, kt_last = p_last / PF_BN;
+    const int n_head = kf > 0 ? min((kf + PF_BN - 1) / PF_BN, kt_first) : 0;
+    const int vt_last = n_head + kt_last - kt_first;
+    auto tile_of = [&](int vt) { return vt < n_head ? vt : vt - n_head + kt_first; };
     // (shaped scores are in base 2 already when they meet the exponent)
     const float sl = SHAPED ? 1.f : scale_log2e;
     // The sequence's block table goes to LDS first: the gathers below then depend on an LDS read,
@@ -140,12 +148,18 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
     u32x4 bk[KPT], bv[KPT];      // register set b: tiles of odd order
     const int ch = tid % CH, grp = tid / CH;
     const int g_lo = k_lo & ~(KPT - 1), g_hi = p_last & ~(KPT - 1);      // first keys of the groups that hold k_lo and p_last
-    auto fetch = [&](u32x4 (&rk)[KPT], u32x4 (&rv)[KPT], int kt) {
-        const int g0 = min(max(kt * PF_BN + grp * KPT, g_lo), g_hi);
+    auto fetch = [&](u32x4 (&rk)[KPT], u32x4 (&rv)[KPT], int vt) {
+        // (a group that holds a kept key lies in a page that is held: it is loaded where it is, its keys between the
+        // kept ones and the window from the last kept key instead)
+        const int G0 = tile_of(vt) * PF_BN + grp * KPT;
+        const bool kept_grp = G0 < kf;
+        const int g0 = min(kept_grp ? G0 : max(G0, g_lo), g_hi);
         const size_t base = page_row(g0) * kv_dim + kv_col + 8 * ch;
 #pragma unroll
         for (int u = 0; u < KPT; ++u) {
-            const int off = (min(max(g0 + u, k_lo), p_last) - g0) * kv_dim;     // stays inside the group
+            const int jj = g0 + u;
+            const int jc = kept_grp ? (jj < kf ? jj : (jj < k_lo ? kf - 1 : jj)) : max(jj, k_lo);
+            const int off = (min(jc, p_last) - g0) * kv_dim;     // stays inside the group
             rk[u] = *reinterpret_cast<const u32x4*>(k_pages + base + off);
             rv[u] = *reinterpret_cast<const u32x4*>(v_pages + base + off);
         }
@@ -175,9 +189,9 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
     // Positions of this wavefront's first and last query: a key tile that every one of them sees
     // in full needs no mask.
     const int pw_min = start + q0 + wave * 16, pw_max = pw_min + 15;
-    auto compute = [&](int kt, int buf, auto masked_tag) {
+    auto compute = [&](int vt, int buf, auto masked_tag) {
         constexpr bool MASKED = decltype(masked_tag)::value;
-        const int j_base = kt * PF_BN;
+        const int j_base = tile_of(vt) * PF_BN;
         const bf16_t* Ks = Ks2[buf];
         const bf16_t* Vt = Vt2[buf];
         // S^T: s[nt][r] is the score of key j_base + 16*(nt0+nt) + 4*G + r with this lane's query
@@ -200,7 +214,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
                     const float z = mllm_shaped_score<true>(acc[r] * scale, shape, r1, r2, max(p - j, 0)) + sbias;
                     float w = __builtin_amdgcn_rcpf(1.f + fast_exp2(-z * MLLM_LOG2E));
                     if (MASKED) {
-                        const bool seen = q_ok && j <= p && (window <= 0 || j > p - window) && (chunk <= 0 || j >= p - p % chunk);
+                        const bool seen = q_ok && j <= p && (window <= 0 || j > p - window || j < kf) && (chunk <= 0 || j >= p - p % chunk);
                         if (!seen) w = 0.f;
                     }
                     s[nt][r] = w;
@@ -208,7 +222,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
                 }
                 if (SHAPED) s[nt][r] = mllm_shaped_score<true>(acc[r] * scale, shape, r1, r2, max(p - j, 0)) * MLLM_LOG2E;
                 if (MASKED) {
-                    const bool seen = q_ok && j <= p && (window <= 0 || j > p - window) && (chunk <= 0 || j >= p - p % chunk);
+                    const bool seen = q_ok && j <= p && (window <= 0 || j > p - window || j < kf) && (chunk <= 0 || j >= p - p % chunk);
                     if (!seen) s[nt][r] = -INFINITY;
                 }
                 tile_max = fmaxf(tile_max, s[nt][r]);
@@ -259,50 +273,49 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
         }
     };
 
-    auto run_tile = [&](int kt, int buf) {
-        const int j_base = kt * PF_BN;
-        const bool full = j_base + PF_BN - 1 <= pw_min && (window <= 0 || j_base > pw_max - window) &&
+    auto run_tile = [&](int vt, int buf) {
+        const int j_base = tile_of(vt) * PF_BN;
+        const bool full = j_base + PF_BN - 1 <= pw_min && (window <= 0 || j_base > pw_max - window || j_base + PF_BN - 1 < kf) &&
                           (chunk <= 0 || j_base >= pw_max - pw_max % chunk);
-        if (full) compute(kt, buf, std::false_type{}); else compute(kt, buf, std::true_type{});
+        if (full) compute(vt, buf, std::false_type{}); else compute(vt, buf, std::true_type{});
     };
 
     // Tile t is multiplied from LDS buffer t % 2 while tile t+1 is written to the other buffer: one barrier
     // per tile. The loop body has no branch around a load; past the last tile the fetches repeat clamped
     // keys, which are staged and never multiplied.
-    const int kt_first = k_lo / PF_BN, kt_last = p_last / PF_BN;
     if constexpr (NW == 8) {
         // Two register sets, every tile requested two tiles ahead of its staging: with half a tile's
         // arithmetic per wavefront, one tile ahead is not enough and the loop runs at the latency of the
         // gather (measured).
-        fetch(ak, av, kt_first);
+        fetch(ak, av, 0);
         __builtin_amdgcn_sched_barrier(0);     // set a's loads stay the older ones, as on every later iteration
-        fetch(bk, bv, kt_first + 1);
+        fetch(bk, bv, 1);
         stage(ak, av, 0);
-        fetch(ak, av, kt_first + 2);
+        fetch(ak, av, 2);
         lds_barrier();
-        for (int kt = kt_first; kt <= kt_last; kt += 2) {
+        for (int vt = 0; vt <= vt_last; vt += 2) {
             stage(bk, bv, 1);                  // (its last readers passed the barrier that ended the tile before)
-            fetch(bk, bv, kt + 3);
-            run_tile(kt, 0);
+            fetch(bk, bv, vt + 3);
+            run_tile(vt, 0);
             lds_barrier();
             stage(ak, av, 0);
-            fetch(ak, av, kt + 4);
-            if (kt + 1 <= kt_last) run_tile(kt + 1, 1);
+            fetch(ak, av, vt + 4);
+            if (vt + 1 <= vt_last) run_tile(vt + 1, 1);
             lds_barrier();
         }
     } else {
         // One register set, requested one tile ahead: a whole tile's arithmetic covers the gather, and the
         // registers saved keep more of the softmax's values out of the way (measured: 28.8 against 31.0 us
         // at 25 heads).
-        fetch(ak, av, kt_first);
+        fetch(ak, av, 0);
         stage(ak, av, 0);
-        fetch(ak, av, kt_first + 1);
+        fetch(ak, av, 1);
         lds_barrier();
-        for (int kt = kt_first; kt <= kt_last; ++kt) {
-            const int buf = (kt - kt_first) & 1;
+        for (int vt = 0; vt <= vt_last; ++vt) {
+            const int buf = vt & 1;
             stage(ak, av, buf ^ 1);
-            fetch(ak, av, kt + 2);
-            run_tile(kt, buf);
+            fetch(ak, av, vt + 2);
+            run_tile(vt, buf);
             lds_barrier();
         }
     }
@@ -331,9 +344,20 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) o[dt][r] = o[dt][r] * a0 + state[2 + 4 * dt + r] * a1;
+        m = m_new;                             // (what the sum and the outputs are now relative to: the sink below reads it)
     }
     l = rows_sum(l);
     if (!q_ok) return;
+    if (SHAPED && !SIGMOID && shape.sink != nullptr) {
+        // the sink: one more term of the denominator, exp(sink), without a value (the maximum is in base 2)
+        const float sk = shape.sink[blockIdx.x] * MLLM_LOG2E, m_new = fmaxf(m, sk);
+        const float a = fast_exp2(m - m_new);
+        l = l * a + fast_exp2(sk - m_new);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[dt][r] *= a;
+    }
     const float inv = SIGMOID ? 1.f : 1.0f / l;
     const bool head_gate = SHAPED && gate != nullptr && shape.gate_per_head;
     const float hg = head_gate ? 1.f / (1.f + __expf(-gate[static_cast<size_t>(q_begin + qi) * ldg + blockIdx.x])) : 1.f;

@@ -22,6 +22,20 @@ void* mllm_cache_create(int n_groups, const int* page_size, const int* n_pages, 
     if (n_state_slots < 0) return nullptr;
     return new CacheManager(groups, n_state_slots);
 }
+// The same with, per group, the number of first keys whose pages a window never gives back early.
+void* mllm_cache_create_keeping(int n_groups, const int* page_size, const int* n_pages, const int* window, const int* keep_first,
+                                int n_state_slots) {
+    std::vector<GroupSpec> groups(n_groups);
+    for (int g = 0; g < n_groups; ++g) {
+        if (page_size[g] < 1 || n_pages[g] < 0 || window[g] < 0 || keep_first[g] < 0) return nullptr;
+        groups[g].page_size = page_size[g];
+        groups[g].n_pages = n_pages[g];
+        groups[g].window = window[g];
+        groups[g].keep_first = keep_first[g];
+    }
+    if (n_state_slots < 0) return nullptr;
+    return new CacheManager(groups, n_state_slots);
+}
 void mllm_cache_destroy(void* c) { delete static_cast<CacheManager*>(c); }
 int mllm_cache_add_request(void* c, int64_t id) { return static_cast<CacheManager*>(c)->add_request(id); }
 int mllm_cache_has_request(void* c, int64_t id) { return static_cast<CacheManager*>(c)->has_request(id) ? 1 : 0; }

@@ -144,8 +144,9 @@ def conv_attention_mixer(h, w, pre, m, eps):
     one more term exp(0) in the denominator."""
     T = h.shape[0]
     H, G, d = m["heads"], m["kv_heads"], m["dim"]
-    q = causal_convolution(project(h, w, pre + "q", False), w[pre + "q.conv"])
-    k = causal_convolution(project(h, w, pre + "k", False), w[pre + "k.conv"])
+    q, k = project(h, w, pre + "q", False), project(h, w, pre + "k", False)
+    if m.get("conv"):
+        q, k = causal_convolution(q, w[pre + "q.conv"]), causal_convolution(k, w[pre + "k.conv"])
     v = k.view(T, G, d)
     q, k = q.view(T, H, d), k.view(T, G, d)
     pos = list(range(T))
