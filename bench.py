@@ -113,7 +113,40 @@ def viladra_config(n_layer, size="gpt2-small", n_positions=1024):
             "vocab_size": 50257, "n_positions": n_positions, "n_layer": n}
 
 
-DESIGNS = {"kugulorn": kugulorn_config, "rekirax": rekirax_config, "viladra": viladra_config}
+def sunulorn_config(n_layer, size="gpt2-small", n_positions=1024):
+    """A Sunulorn model with as many layers as the GPT-2 configuration `size` has, at the same width, vocabulary and
+    context: its three attentions in turn (a convolution of four taps over queries and keys with 32 interleaved rotated
+    columns; a window of 512 that keeps the first 16 positions, all 64 columns rotated; a distance penalty, a sink and
+    a gate per head, every second such layer reading the keys and values of the one before it), heads of 64 as many as
+    GPT-2 has and a quarter as many key/value heads; a gated feed-forward and eight clamped gated experts of which two
+    are chosen beside a shared one in turn, each holding what GPT-2's two feed-forward matrices do."""
+    full_layers, d, h, f = SIZES[size]
+    n = n_layer or full_layers
+    kv = max(k for k in range(1, max(h // 4, 1) + 1) if h % k == 0)
+    dense = {"kind": "dense", "ff": f * 2 // 3 // 64 * 64}
+    moe = {"kind": "moe", "router": {"experts": 8, "top": 2}, "expert": {"ff": f // 16, "limit": 7.0}, "shared": {"ff": f // 6 // 64 * 64, "limit": 7.0}}
+    layers, last_own = [], None
+    for i in range(n):
+        mlp = dense if i % 2 == 0 else moe
+        base = {"heads": h, "kv_heads": kv, "dim": 64, "vdim": 64, "scale": 0.125}
+        if i % 3 == 0:
+            layers.append({"type": "attention", "mlp": mlp, "mixer": dict(base, conv=4, rot={"base": 10000.0, "dims": 32})})
+        elif i % 3 == 1:
+            layers.append({"type": "attention_2", "mlp": mlp,
+                           "mixer": dict(base, rot={"base": 10000.0, "dims": 64}, mask={"size": 512, "keep_first": 16})})
+        else:
+            m = dict(base)
+            if last_own is not None and (i // 3) % 2 == 1:
+                m["kv_from"] = last_own
+            else:
+                last_own = i
+            layers.append({"type": "attention_3", "mlp": mlp, "mixer": m})
+    return {"architecture": "Sunulorn", "vocab": 50257, "width": d, "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0}, "layers": layers,
+            # (what the measurement itself reads; the architecture ignores them)
+            "vocab_size": 50257, "n_positions": n_positions, "n_layer": n}
+
+
+DESIGNS = {"kugulorn": kugulorn_config, "rekirax": rekirax_config, "viladra": viladra_config, "sunulorn": sunulorn_config}
 
 
 def decode_run(model_dir, dtype, batch, prompt_len, steps, warmup, cfg):
@@ -347,10 +380,10 @@ def main():
     ap.add_argument("--config", help="a config.json to measure in place of the GPT-2 sizes (any registered architecture; "
                                      "it names vocab_size and n_positions, or --vocab / --positions do)")
     ap.add_argument("--vocab", type=int, default=0, help="with --config: the vocabulary to draw token ids from")
-    ap.add_argument("--design", default="gpt2", choices=["gpt2", "kugulorn", "rekirax", "viladra"],
-                    help="kugulorn / rekirax / viladra: a model of that design of about the size --size names (kugulorn_config, "
-                         "rekirax_config, viladra_config) through the same measurement; --compare runs it and GPT-2 one after the other")
-    ap.add_argument("--beside", default="gpt2", choices=["gpt2", "kugulorn", "rekirax", "viladra"],
+    ap.add_argument("--design", default="gpt2", choices=["gpt2", "kugulorn", "rekirax", "viladra", "sunulorn"],
+                    help="kugulorn / rekirax / viladra / sunulorn: a model of that design of about the size --size names (kugulorn_config, "
+                         "rekirax_config, viladra_config, sunulorn_config) through the same measurement; --compare runs it and GPT-2 one after the other")
+    ap.add_argument("--beside", default="gpt2", choices=["gpt2", "kugulorn", "rekirax", "viladra", "sunulorn"],
                     help="with --compare: the design that the --design model is measured beside (default GPT-2)")
     ap.add_argument("--compare", action="store_true",
                     help="prefill (2 x 1,024 tokens) and decode (batch 1, 8, 64) of the --design model (default Kugulorn) and of the GPT-2 model "

@@ -84,10 +84,10 @@ int mllm_fill_zero(void* p, size_t bytes, hipStream_t stream);
 // ssm.hip
 int mllm_conv_silu(const float* proj, int ld, int col0, int C, const float* w, const float* bias, int taps,
                    const int* token_seq, const int* cu_q, const int* state_slots, float* state, size_t slot_floats,
-                   float* out, int ldo, int T, int B, int write, hipStream_t stream, int activation = 1);
+                   float* out, int ldo, int T, int B, int write, hipStream_t stream);
 int mllm_conv_residual(const float* in, int ld, int C, const float* w, int taps, const int* token_seq, const int* cu_q,
                        const int* state_slots, float* state, size_t slot_floats, void* out, int ldo, int out_dtype, int T,
-                       int B, int write, hipStream_t stream);
+                       int B, int write, hipStream_t stream, int residual = 1);
 int mllm_rmsnorm_conv_single(const float* x, int ldx, const float* wn, float eps, int C, const float* wc, int taps,
                              const int* state_slots, float* state, size_t slot_floats, void* out, int ldo, int out_dtype, int T,
                              int write, hipStream_t stream);

@@ -196,9 +196,8 @@ struct StateArgs {
 };
 // out[t, :] = silu(conv(columns [col0, col0 + C) of proj)), causal per sequence over `taps` inputs, the inputs
 // before a portion taken from the slot's first (taps - 1) * C floats, which are brought up to date afterwards.
-// With `silu` false the convolution stands alone: no activation, and the bias may be null.
 void conv_silu(const Tensor2& proj, int col0, const Tensor2& weight, const float* bias, const StateArgs& st,
-               const Tensor2& out, hipStream_t stream, bool silu = true);
+               const Tensor2& out, hipStream_t stream);
 // The Mamba-2 scan (kernels/ssm.hip) over xbc [T, H*P + 2*G*N] and the raw step sizes (columns dt_col.. of
 // proj), state at `scan_offset` floats into the slot. y comes as ssm_scan_parts(N) shares, each [T, H*P] fp32
 // and y.rows * y.stride floats after the one before (y is the first); their sum in the order of their index is
@@ -251,7 +250,8 @@ void latent_expand(const Tensor2& o_lat, const Tensor2& w_uv, const Tensor2& out
 // -- attention with shaped scores -------------------------------------------------------------------
 // out = in + conv(in): a causal convolution per channel over `taps` inputs (taps [channels, taps], the last tap
 // the token's own), added onto its input; in fp32 [T, C], out in its own dtype. Carried inputs as for conv_silu.
-void conv_residual(const Tensor2& in, const Tensor2& weight, const StateArgs& st, const Tensor2& out, hipStream_t stream);
+// With `residual` false the input is not added: out = conv(in) alone.
+void conv_residual(const Tensor2& in, const Tensor2& weight, const StateArgs& st, const Tensor2& out, hipStream_t stream, bool residual = true);
 // The same behind an RMS norm, in one kernel, for a step in which every sequence brings one token (x.rows == st.n_seqs):
 // out = h + conv(h) with h = x / sqrt(mean(x^2) + eps) * norm_weight.
 // False (and nothing done): sizes the kernel is not made for (more than 8 taps, rows wider than 2,048).

@@ -40,7 +40,7 @@ void check_shape(const ScoredShape& sh, const char* what) {
 }
 }  // namespace
 
-void conv_residual(const Tensor2& in, const Tensor2& weight, const StateArgs& st, const Tensor2& out, hipStream_t stream) {
+void conv_residual(const Tensor2& in, const Tensor2& weight, const StateArgs& st, const Tensor2& out, hipStream_t stream, bool residual) {
     need_f32(in, "conv_residual: the input");
     need_f32(weight, "conv_residual: the taps");
     need_act(out, "conv_residual: out");
@@ -53,7 +53,7 @@ void conv_residual(const Tensor2& in, const Tensor2& weight, const StateArgs& st
         fail("conv_residual: the step's token_seq, cu_q and state slots are needed");
     check(mllm_conv_residual(static_cast<const float*>(in.data), i32(in.stride), C, static_cast<const float*>(weight.data), taps, st.token_seq,
                              st.cu_q, st.state_slots, st.state, st.slot_floats, out.data, i32(out.stride), out.dtype, i32(in.rows), st.n_seqs,
-                             st.write ? 1 : 0, stream), "conv_residual");
+                             st.write ? 1 : 0, stream, residual ? 1 : 0), "conv_residual");
 }
 
 bool rmsnorm_conv_single(const Tensor2& x, const float* norm_weight, float eps, const Tensor2& weight, const StateArgs& st,

@@ -102,23 +102,20 @@ void fill_zero(const Tensor2& x, hipStream_t stream) {
 }
 
 void conv_silu(const Tensor2& proj, int col0, const Tensor2& weight, const float* bias, const StateArgs& st,
-               const Tensor2& out, hipStream_t stream, bool silu) {
+               const Tensor2& out, hipStream_t stream) {
     need_f32(proj, "conv_silu: the input");
     need_f32(out, "conv_silu: out");
     need_f32(weight, "conv_silu: the taps");
     const int C = i32(weight.rows), taps = i32(weight.cols);
-    if (!weight.contiguous() || (silu && bias == nullptr)) fail("conv_silu: taps [channels, taps] contiguous and a bias are needed");
+    if (!weight.contiguous() || bias == nullptr) fail("conv_silu: taps [channels, taps] contiguous and a bias are needed");
     if (taps < 1 || taps > 16) fail("conv_silu: %d taps are not supported (1 to 16)", taps);
     if (col0 < 0 || col0 + C > proj.cols || out.cols != C || out.rows != proj.rows)
         fail("conv_silu: %d channels from column %d do not fit rows of %lld, or out is not [%lld, %d]", C, col0, (long long)proj.cols,
              (long long)proj.rows, C);
-    // (a single tap reads no carried rows: such a convolution needs no state, only the step's arrays)
-    if (taps > 1) check_state(st, static_cast<size_t>(taps - 1) * C, "conv_silu");
-    else if (st.token_seq == nullptr || st.cu_q == nullptr || st.state_slots == nullptr || st.n_seqs < 1)
-        fail("conv_silu: the step's token_seq, cu_q and state slots are needed");
+    check_state(st, static_cast<size_t>(taps - 1) * C, "conv_silu");
     check(mllm_conv_silu(static_cast<const float*>(proj.data), i32(proj.stride), col0, C, static_cast<const float*>(weight.data), bias, taps,
                          st.token_seq, st.cu_q, st.state_slots, st.state, st.slot_floats, static_cast<float*>(out.data), i32(out.stride),
-                         i32(proj.rows), st.n_seqs, st.write ? 1 : 0, stream, silu ? 1 : 0), "conv_silu");
+                         i32(proj.rows), st.n_seqs, st.write ? 1 : 0, stream), "conv_silu");
 }
 
 void ssm_scan(const Tensor2& xbc, const Tensor2& proj, int dt_col, const float* dt_bias, const float* A_log,

@@ -130,7 +130,7 @@ public:
             st.token_seq = step.token_seq; st.cu_q = step.cu_q; st.state_slots = step.state_slots; st.n_seqs = step.n_seqs;
             st.max_q_len = step.max_q_len; st.state = static_cast<float*>(cache.state); st.slot_floats = cache.slot_bytes / 4;
             st.n_slots = cache.n_slots; st.write = write;
-            conv_silu(proj, 0, conv_, nullptr, st, qk, s, false);
+            conv_residual(Tensor2(proj.data, F32, T, C, ld), conv_, st, qk, s, false);      // (four channels a thread where the sizes allow)
             qk_prepare(qk, 0, k_col_, v_col_, sh_, step.positions, step.slots[g], q, cache.k_pages, cache.v_pages, s);
         } else {
             qk_prepare(proj, 0, k_col_, v_col_, sh_, step.positions, step.slots[g], q, cache.k_pages, cache.v_pages, s);

@@ -37,8 +37,10 @@ __device__ __forceinline__ void expert_weight(const float* z, float* wgt, int E,
 // on the expert's INPUT, which a linear map hands on to its result; `weight_on_input` 0: g and u unweighted and the
 // weight on the result) out[t, e * ff + j] = g sigmoid(alpha g) (u + 1), zero for an expert that was not chosen. The
 // shared expert's columns follow, unweighted, with its own limit, times sigmoid(logits[t, E]) if `shared_gate` (the
-// router's product then has one more row). One workgroup per token.
-template <typename T>
+// router's product then has one more row). One workgroup per token. VEC: eight columns a thread at a time (16-byte
+// loads of bfloat16, two of float; ff, shared_ff and the strides are then multiples of 8 and the rows aligned), all of
+// one expert.
+template <typename T, bool VEC>
 __global__ void __launch_bounds__(256)
 moe_glu_act_kernel(const T* __restrict__ up, int ldu, const float* __restrict__ logits, int ldl, int E, int ff, int shared_ff, int top,
                    float scale, int sigmoid_router, float limit, float shared_limit, float alpha, int weight_on_input, int shared_gate,
@@ -54,6 +56,42 @@ moe_glu_act_kernel(const T* __restrict__ up, int ldu, const float* __restrict__ 
     const T* ur = up + static_cast<size_t>(t) * ldu;
     T* orow = out + static_cast<size_t>(t) * ldo;
     const int routed = E * ff, N = routed + shared_ff;
+    if (VEC) {
+        for (int c = tid * 8; c < N; c += 256 * 8) {
+            float g[8], u[8], lim, w_in = 1.f, w_out = 1.f;
+            bool live = true;
+            if (c < routed) {
+                const int e = c / ff, j = c - e * ff;
+                load8(ur + static_cast<size_t>(e) * 2 * ff + j, g);
+                load8(ur + static_cast<size_t>(e) * 2 * ff + ff + j, u);
+                lim = limit;
+                live = wgt[e] != 0.f;
+                if (weight_on_input) w_in = wgt[e]; else w_out = wgt[e];
+            } else {
+                const int j = c - routed;
+                load8(ur + static_cast<size_t>(routed) * 2 + j, g);
+                load8(ur + static_cast<size_t>(routed) * 2 + shared_ff + j, u);
+                lim = shared_limit;
+                w_out = sg_s;
+            }
+            float y[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const float gk = fminf(g[k] * w_in, lim), uk = fminf(fmaxf(u[k] * w_in, -lim), lim);
+                const float ex = sizeof(T) == 2 ? __expf(-alpha * gk) : expf(-alpha * gk);
+                y[k] = live ? gk / (1.f + ex) * (uk + 1.f) * w_out : 0.f;
+            }
+            if (sizeof(T) == 2) {
+                uint4 pk;
+                pk.x = pack_bf16x2(y[0], y[1]); pk.y = pack_bf16x2(y[2], y[3]); pk.z = pack_bf16x2(y[4], y[5]); pk.w = pack_bf16x2(y[6], y[7]);
+                *reinterpret_cast<uint4*>(orow + c) = pk;
+            } else {
+                *reinterpret_cast<float4*>(orow + c) = make_float4(y[0], y[1], y[2], y[3]);
+                *reinterpret_cast<float4*>(orow + c + 4) = make_float4(y[4], y[5], y[6], y[7]);
+            }
+        }
+        return;
+    }
     for (int c = tid; c < N; c += 256) {
         float g, u, lim, w_in = 1.f, w_out = 1.f;
         bool live = true;
@@ -157,12 +195,15 @@ int mllm_moe_glu_act(const void* up, int ldu, const float* logits, int ldl, int 
     if (T <= 0) return 0;
     if (E < 1 || E > MOE_MAX_EXPERTS || top < 1 || top > E || ff < 1 || shared_ff < 0 || logits == nullptr) return -1;
     if (!(limit > 0.f) || (shared_ff > 0 && !(shared_limit > 0.f)) || (shared_gate && shared_ff == 0)) return -1;
-    if (dtype == MLLM_F32)
-        moe_glu_act_kernel<float><<<T, 256, 0, stream>>>(static_cast<const float*>(up), ldu, logits, ldl, E, ff, shared_ff, top, scale, sigmoid_router,
-                                                        limit, shared_limit, alpha, weight_on_input, shared_gate, static_cast<float*>(out), ldo);
-    else
-        moe_glu_act_kernel<bf16_t><<<T, 256, 0, stream>>>(static_cast<const bf16_t*>(up), ldu, logits, ldl, E, ff, shared_ff, top, scale, sigmoid_router,
-                                                         limit, shared_limit, alpha, weight_on_input, shared_gate, static_cast<bf16_t*>(out), ldo);
+    const int esz = dtype == MLLM_F32 ? 4 : 2;
+    const bool vec = ff % 8 == 0 && shared_ff % 8 == 0 && ldu % 8 == 0 && ldo % 8 == 0 &&
+                     ((reinterpret_cast<uintptr_t>(up) | reinterpret_cast<uintptr_t>(out)) & 15) == 0 && (static_cast<size_t>(ldu) * esz) % 16 == 0;
+#define MOE_GLU(TYPE, VEC)                                                                                                                     \
+    moe_glu_act_kernel<TYPE, VEC><<<T, 256, 0, stream>>>(static_cast<const TYPE*>(up), ldu, logits, ldl, E, ff, shared_ff, top, scale, sigmoid_router, \
+                                                         limit, shared_limit, alpha, weight_on_input, shared_gate, static_cast<TYPE*>(out), ldo)
+    if (dtype == MLLM_F32) { if (vec) MOE_GLU(float, true); else MOE_GLU(float, false); }
+    else { if (vec) MOE_GLU(bf16_t, true); else MOE_GLU(bf16_t, false); }
+#undef MOE_GLU
     MLLM_LAUNCH_CHECK();
     return 0;
 }

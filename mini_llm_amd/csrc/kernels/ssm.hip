@@ -16,8 +16,6 @@ __device__ __forceinline__ float softplus_precise(float v) { return fmaxf(v, 0.f
 
 // out[t, ch] = silu(bias[ch] + sum_j w[ch, j] * in(t - (taps - 1 - j), ch)): inputs before the portion come
 // from the slot's carried rows (zeros for a fresh request: the slot was cleared). One thread per (t, ch).
-// SILU false: the convolution alone, no activation; the bias may be null.
-template <bool SILU>
 __global__ void conv_silu_kernel(const float* __restrict__ proj, int ld, int col0, int C, const float* __restrict__ w,
                                  const float* __restrict__ bias, int taps, const int* __restrict__ token_seq,
                                  const int* __restrict__ cu_q, const int* __restrict__ state_slots,
@@ -30,7 +28,7 @@ __global__ void conv_silu_kernel(const float* __restrict__ proj, int ld, int col
     if (slot < 0) return;
     const int first = cu_q[b], k = t - first;
     float* carried = state + static_cast<size_t>(slot) * slot_floats;
-    float acc = bias != nullptr ? bias[ch] : 0.f;
+    float acc = bias[ch];
     for (int j = 0; j < taps; ++j) {
         const int idx = k - (taps - 1 - j);
         const float v = idx >= 0 ? proj[static_cast<size_t>(first + idx) * ld + col0 + ch]
@@ -40,16 +38,17 @@ __global__ void conv_silu_kernel(const float* __restrict__ proj, int ld, int col
         // carried rows move up by one behind the read, and the token's input becomes the newest
         if (carry && j >= 1) carried[static_cast<size_t>(j - 1) * C + ch] = v;
     }
-    out[static_cast<size_t>(t) * ldo + ch] = SILU ? silu_precise(acc) : acc;
+    out[static_cast<size_t>(t) * ldo + ch] = silu_precise(acc);
 }
 
 // out[t, ch] = in[t, ch] + sum_j w[ch, j] * in(t - (taps - 1 - j), ch): the convolution added onto its own input,
-// no bias and no activation, the result in the activation dtype. Carried rows as above.
+// no bias and no activation, the result in the activation dtype. Carried rows as above. residual == 0: the
+// convolution alone, its input not added.
 template <typename OutT>
 __global__ void conv_residual_kernel(const float* __restrict__ in, int ld, int C, const float* __restrict__ w, int taps,
                                      const int* __restrict__ token_seq, const int* __restrict__ cu_q,
                                      const int* __restrict__ state_slots, float* __restrict__ state, size_t slot_floats,
-                                     OutT* __restrict__ out, int ldo, long long total, int carry) {
+                                     OutT* __restrict__ out, int ldo, long long total, int carry, int residual) {
     const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= total) return;
     const int t = static_cast<int>(i / C), ch = static_cast<int>(i % C);
@@ -66,7 +65,7 @@ __global__ void conv_residual_kernel(const float* __restrict__ in, int ld, int C
         own = v;
         if (carry && j >= 1) carried[static_cast<size_t>(j - 1) * C + ch] = v;
     }
-    out[static_cast<size_t>(t) * ldo + ch] = from_float<OutT>(own + acc);
+    out[static_cast<size_t>(t) * ldo + ch] = from_float<OutT>(residual ? own + acc : acc);
 }
 
 // The same four channels a thread (16-byte loads; the rows' widths and the places are multiples of four floats). A
@@ -81,7 +80,7 @@ template <typename OutT, int TAPS>
 __global__ void conv_residual_vec_kernel(const float* __restrict__ in, int ld, int C, const float* __restrict__ w,
                                          const int* __restrict__ token_seq, const int* __restrict__ cu_q,
                                          const int* __restrict__ state_slots, float* __restrict__ state, size_t slot_floats,
-                                         OutT* __restrict__ out, int ldo, long long total4, int carry) {
+                                         OutT* __restrict__ out, int ldo, long long total4, int carry, int residual) {
     const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= total4) return;
     const int C4 = C / 4;
@@ -108,6 +107,7 @@ __global__ void conv_residual_vec_kernel(const float* __restrict__ in, int ld, i
 #pragma unroll
     for (int j = 0; j < TAPS; ++j) { wv[4 * j] = wf[j].x; wv[4 * j + 1] = wf[j].y; wv[4 * j + 2] = wf[j].z; wv[4 * j + 3] = wf[j].w; }
     float r[4] = {v[TAPS - 1].x, v[TAPS - 1].y, v[TAPS - 1].z, v[TAPS - 1].w};
+    if (!residual) r[0] = r[1] = r[2] = r[3] = 0.f;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int j = 0; j < TAPS; ++j) {
@@ -575,24 +575,19 @@ static int stream_conv_single_launch(float* x, int ldx, const float* y, int ldy,
 
 extern "C" {
 
-// Convolution + silu (activation 0: the convolution alone, the bias may be null) of columns [col0, col0 + C) of
-// proj's rows into out [T, C]; then, with `write`, the
+// Convolution + silu of columns [col0, col0 + C) of proj's rows into out [T, C]; then, with `write`, the
 // slots' carried rows are brought up to date (a second kernel: it overwrites what the first one reads).
 // -1: taps outside 1..16.
 int mllm_conv_silu(const float* proj, int ld, int col0, int C, const float* w, const float* bias, int taps,
                    const int* token_seq, const int* cu_q, const int* state_slots, float* state, size_t slot_floats,
-                   float* out, int ldo, int T, int B, int write, hipStream_t stream, int activation) {
+                   float* out, int ldo, int T, int B, int write, hipStream_t stream) {
     if (T <= 0 || C <= 0) return 0;
-    if (taps < 1 || taps > 16 || (activation != 0 && bias == nullptr)) return -1;
+    if (taps < 1 || taps > 16) return -1;
     const long long total = static_cast<long long>(T) * C;
     // (one token a sequence: the convolution's kernel brings the carried rows up to date itself)
     const bool single = T == B && write && taps > 1;
-    if (activation != 0)
-        conv_silu_kernel<true><<<static_cast<int>((total + 255) / 256), 256, 0, stream>>>(proj, ld, col0, C, w, bias, taps, token_seq, cu_q,
-                                                                                          state_slots, state, slot_floats, out, ldo, total, single ? 1 : 0);
-    else
-        conv_silu_kernel<false><<<static_cast<int>((total + 255) / 256), 256, 0, stream>>>(proj, ld, col0, C, w, bias, taps, token_seq, cu_q,
-                                                                                           state_slots, state, slot_floats, out, ldo, total, single ? 1 : 0);
+    conv_silu_kernel<<<static_cast<int>((total + 255) / 256), 256, 0, stream>>>(proj, ld, col0, C, w, bias, taps, token_seq, cu_q,
+                                                                                state_slots, state, slot_floats, out, ldo, total, single ? 1 : 0);
     MLLM_LAUNCH_CHECK();
     if (write && taps > 1 && !single) {
         const long long pairs = static_cast<long long>(B) * C;
@@ -603,11 +598,11 @@ int mllm_conv_silu(const float* proj, int ld, int col0, int C, const float* w, c
     return 0;
 }
 
-// out = in + conv(in) over the C columns of in's rows (fp32), out in out_dtype; the slots' carried rows are brought
-// up to date as by mllm_conv_silu. -1: taps outside 1..16.
+// out = in + conv(in) (residual == 0: conv(in) alone) over the C columns of in's rows (fp32), out in out_dtype; the
+// slots' carried rows are brought up to date as by mllm_conv_silu. -1: taps outside 1..16.
 int mllm_conv_residual(const float* in, int ld, int C, const float* w, int taps, const int* token_seq, const int* cu_q,
                        const int* state_slots, float* state, size_t slot_floats, void* out, int ldo, int out_dtype, int T,
-                       int B, int write, hipStream_t stream) {
+                       int B, int write, hipStream_t stream, int residual) {
     if (T <= 0 || C <= 0) return 0;
     if (taps < 1 || taps > 16) return -1;
     const long long total = static_cast<long long>(T) * C;
@@ -620,7 +615,7 @@ int mllm_conv_residual(const float* in, int ld, int C, const float* w, int taps,
         const int blocks4 = static_cast<int>((total4 + 255) / 256);
 #define CRV(TYPE, TAPS)                                                                                                \
     conv_residual_vec_kernel<TYPE, TAPS><<<blocks4, 256, 0, stream>>>(in, ld, C, w, token_seq, cu_q, state_slots, state, slot_floats, \
-                                                                     static_cast<TYPE*>(out), ldo, total4, single ? 1 : 0)
+                                                                     static_cast<TYPE*>(out), ldo, total4, single ? 1 : 0, residual)
 #define CRV_TAPS(TYPE)                                                                                                 \
     switch (taps) {                                                                                                    \
         case 1: CRV(TYPE, 1); break; case 2: CRV(TYPE, 2); break; case 3: CRV(TYPE, 3); break; case 4: CRV(TYPE, 4); break; \
@@ -633,10 +628,10 @@ int mllm_conv_residual(const float* in, int ld, int C, const float* w, int taps,
         const int blocks = static_cast<int>((total + 255) / 256);
         if (out_dtype == MLLM_F32)
             conv_residual_kernel<float><<<blocks, 256, 0, stream>>>(in, ld, C, w, taps, token_seq, cu_q, state_slots, state, slot_floats,
-                                                                    static_cast<float*>(out), ldo, total, single ? 1 : 0);
+                                                                    static_cast<float*>(out), ldo, total, single ? 1 : 0, residual);
         else
             conv_residual_kernel<bf16_t><<<blocks, 256, 0, stream>>>(in, ld, C, w, taps, token_seq, cu_q, state_slots, state,
-                                                                     slot_floats, static_cast<bf16_t*>(out), ldo, total, single ? 1 : 0);
+                                                                     slot_floats, static_cast<bf16_t*>(out), ldo, total, single ? 1 : 0, residual);
     }
     MLLM_LAUNCH_CHECK();
     if (write && taps > 1 && !single) {
