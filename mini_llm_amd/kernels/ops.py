@@ -50,7 +50,9 @@ class AttentionArgsC(ctypes.Structure):
 
 
 class ScoreShapeC(ctypes.Structure):
-    _fields_ = [("softcap", _f), ("chunk", _i), ("r1", _vp), ("r2", _vp), ("sigmoid", _i), ("score_bias", _vp), ("gate_per_head", _i)]
+    # (field for field the kernels' MllmScoreShape, csrc/kernels/score_shape.h)
+    _fields_ = [("softcap", _f), ("chunk", _i), ("r1", _vp), ("r2", _vp), ("sigmoid", _i), ("score_bias", _vp), ("gate_per_head", _i),
+                ("slope", _vp), ("sink", _vp), ("keep_first", _i)]
 
 
 _lib = None
@@ -415,7 +417,7 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
     in place of ``out`` (returned when a few single tokens' keys were split over several workgroups
     each; ``out`` is then left unwritten).
 
-    ``shape``: scores shaped before the softmax, ``{"softcap": c, "chunk": n, "r1": tensor, "r2": tensor}`` (any
+    ``shape``: scores shaped before the softmax, ``{"softcap": c, "chunk": n, "r1": tensor, "r2": tensor, "slope": tensor, "sink": tensor, "keep_first": n}`` (any
     subset): ``s <- c tanh(s / c)``, then ``s <- s - r1[h] ln(1 + r2[h] (i - j))`` (fp32 [n_heads] each), and with
     ``chunk`` a query sees only the keys of its own block of n positions. ``gate`` (fp32 [T, n_heads*head_dim],
     only with ``shape``): the result is multiplied by its sigmoid. Neither goes with ``append`` or ``may_split``.
@@ -466,6 +468,14 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
             if sb.dtype != torch.float32 or sb.numel() != n_heads or not sb.is_contiguous():
                 raise KernelError("score_bias must be contiguous float32 [n_heads]")
             sh.score_bias = sb.data_ptr()
+        for key in ("slope", "sink"):
+            v = shape.get(key)
+            if v is not None:
+                _gpu(v)
+                if v.dtype != torch.float32 or v.numel() != n_heads or not v.is_contiguous():
+                    raise KernelError(f"{key} must be contiguous float32 [n_heads]")
+                setattr(sh, key, v.data_ptr())
+        sh.keep_first = int(shape.get("keep_first") or 0)
         a.shape = ctypes.addressof(sh)
     if gate is not None:
         _gpu(gate)

@@ -36,6 +36,7 @@ static void one_run(unsigned seed) {
     std::vector<GroupSpec> groups(2);
     groups[0].page_size = page; groups[0].n_pages = pick((max_pos + page - 1) / page + 1, 3 * max_pos / page + 2); groups[0].window = 0;
     groups[1].page_size = page; groups[1].n_pages = groups[0].n_pages; groups[1].window = pick(3, 40);
+    groups[1].keep_first = pick(0, 1) ? pick(1, 30) : 0;      // (every second workload: the window also keeps its first keys' pages)
     CacheManager cache(groups, n_slots);
     SchedulerOptions opt;
     opt.max_num_seqs = pick(1, n_slots);

@@ -102,6 +102,9 @@ def paged_attention(q, q_col, n_heads, n_kv_heads, head_dim, k_pages, v_pages, p
         if shape and shape.get("chunk"):
             lo = p - p % shape["chunk"]           # only the keys of the query's own block of positions
         js = torch.arange(lo, p + 1)
+        if shape and shape.get("keep_first") and window:
+            # the sequence's first positions stay visible in front of the window, at their true distances
+            js = torch.cat([torch.arange(0, min(shape["keep_first"], lo)), js])
         rows = block_tables[b].long()[js // page_size] * page_size + js % page_size
         for h in range(n_heads):
             hk = h // rep
@@ -113,10 +116,15 @@ def paged_attention(q, q_col, n_heads, n_kv_heads, head_dim, k_pages, v_pages, p
                 s = shape["softcap"] * torch.tanh(s / shape["softcap"])
             if shape and shape.get("r1") is not None:
                 s = s - shape["r1"][h].to(PRECISE) * torch.log1p(shape["r2"][h].to(PRECISE) * (p - js).to(PRECISE))
+            if shape and shape.get("slope") is not None:
+                s = s - shape["slope"][h].to(PRECISE) * (p - js).to(PRECISE)
             if shape and shape.get("sigmoid"):
                 # every visible key on its own: sigmoid(score + the head's bias), not normalised over the keys
                 bias = shape["score_bias"][h].to(PRECISE) if shape.get("score_bias") is not None else 0.0
                 w = torch.sigmoid(s + bias)
+            elif shape and shape.get("sink") is not None:
+                # one more term in the denominator, exp(sink), that has no value
+                w = torch.softmax(torch.cat([s, shape["sink"][h].to(PRECISE).view(1)]), dim=0)[:-1]
             else:
                 w = torch.softmax(s, dim=0)
             o = w @ v

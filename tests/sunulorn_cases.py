@@ -58,6 +58,7 @@ ONLY_CONV = model([conv_attention()])
 ONLY_CONV_BARE = model([conv_attention(heads=3, kv_heads=3, dim=24, taps=None, dims=None)], width=48, embed_scale=None)   # no convolution, no turn
 ONLY_CONV_ONE_TAP = model([conv_attention(heads=2, kv_heads=1, dim=32, taps=1, dims=32, base=300.0)], width=32)
 ONLY_CONV_LONG = model([conv_attention(heads=2, kv_heads=2, dim=8, taps=7, dims=2)], width=40)
+ONLY_CONV_MANY_TAPS = model([conv_attention(heads=2, kv_heads=1, dim=8, taps=13, dims=4)], width=24)     # more taps than the four-channel kernel takes
 ONLY_WINDOW = model([window_attention()])
 ONLY_WINDOW_NO_KEEP = model([window_attention(heads=3, kv_heads=1, dim=24, vdim=8, window=6, keep=None, dims=8)], width=48)
 ONLY_WINDOW_OPEN = model([window_attention(heads=2, kv_heads=2, dim=16, vdim=16, window=None, dims=None)], width=32)    # plain causal, no turn

@@ -529,7 +529,7 @@ def test_paged_attention_decode_only(ops, dtype, H, Hkv, dh, page, window, shape
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,Hkv,dh,page", [(4, 2, 64, 16), (6, 2, 128, 16), (3, 3, 32, 8), (5, 5, 48, 16), (2, 1, 40, 4)])
-@pytest.mark.parametrize("kind", ["window_bias", "chunk_gate", "sigmoid"])
+@pytest.mark.parametrize("kind", ["window_bias", "chunk_gate", "sigmoid", "slope_sink", "window_keep"])
 def test_paged_attention_with_shaped_scores(ops, dtype, H, Hkv, dh, page, kind):
     """Scores capped and biased by the distance under a sliding window, or a chunked mask with a gate on the result,
     on every kernel of the dispatch: prompt portions (matrix-core tiles in bfloat16 and in 32-bit; the row kernel for
@@ -546,14 +546,26 @@ def test_paged_attention_with_shaped_scores(ops, dtype, H, Hkv, dh, page, kind):
             pytest.skip("sigmoid weights run on these kernels in bfloat16 at head sizes 32, 64, 128")
         window = 150
         shape = {"sigmoid": 1, "score_bias": torch.randn(H, generator=g) - 4.0, "gate_per_head": 1}
+    elif kind == "slope_sink":
+        # a penalty that grows linearly with the distance, a sink per head in the denominator (some as large as the
+        # boosted key's score), a gate per head: every kernel of the dispatch takes them, in both precisions
+        window = 0
+        shape = {"slope": torch.rand(H, generator=g) * 0.02, "sink": torch.randn(H, generator=g) * 3.0 + 2.0, "gate_per_head": 1}
+    elif kind == "window_keep":
+        # a window of 150 that also sees the first 70 positions (more than a key tile of the 32-bit kernel, less than one
+        # of the matrix-core kernel), with a sink
+        window = 150
+        shape = {"keep_first": 70, "sink": torch.randn(H, generator=g)}
     else:
         window = 0
         shape = {"chunk": 70}
-    gated = kind in ("chunk_gate", "sigmoid")
+    gated = kind in ("chunk_gate", "sigmoid", "slope_sink")
     cases = [([(0, 37), (130, 70), (64, 2), (5, 300)], 0), ([(1023, 1), (0, 1), (63, 1), (149, 1), (150, 1), (69, 1), (70, 1), (500, 1)], 8),
              ([(300, 1), (12, 1), (0, 100), (200, 64), (139, 1)], 2)]
     for seqs, n_single in cases:
-        out, ref = _attention_case(ops, dtype, H, Hkv, dh, page, seqs, window, g, boost=(max(0, seqs[0][0] + seqs[0][1] - 3), 0.5),
+        # (kept first positions: the boosted key is one of them, far in front of the last sequence's window)
+        far = 5 if kind == "window_keep" else max(0, seqs[0][0] + seqs[0][1] - 3)
+        out, ref = _attention_case(ops, dtype, H, Hkv, dh, page, seqs, window, g, boost=(far, 0.5),
                                    n_single=n_single, q_col=0, shape=shape, gated=gated)
         assert torch.isfinite(out).all()
         # (sums of weights that are not normalised grow with the keys: relative to the largest value)

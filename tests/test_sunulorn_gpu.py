@@ -43,7 +43,7 @@ def _families(reqs, seed):
             "chunks": ru.trace_chunks(reqs, seed=seed), "mixed": mixed}
 
 
-SINGLE = ["ONLY_CONV", "ONLY_CONV_BARE", "ONLY_CONV_ONE_TAP", "ONLY_CONV_LONG", "ONLY_WINDOW", "ONLY_WINDOW_NO_KEEP",
+SINGLE = ["ONLY_CONV", "ONLY_CONV_BARE", "ONLY_CONV_ONE_TAP", "ONLY_CONV_LONG", "ONLY_CONV_MANY_TAPS", "ONLY_WINDOW", "ONLY_WINDOW_NO_KEEP",
           "ONLY_WINDOW_OPEN", "ONLY_WINDOW_KEEP_WIDE", "ONLY_SINK", "ONLY_SINK_ONE_HEAD", "ONLY_SINK_MANY", "SHARED_KV",
           "ONLY_DENSE", "ONLY_EXPERTS", "ONLY_EXPERTS_ALL", "ONE_EXPERT", "TOP_ONE", "SINK_SOFT"]
 
