@@ -192,22 +192,44 @@ public:
         run(h, step, x, arena, s, STORE_F32);
     }
     void run(NormedInput& h, const StepView& step, const Tensor2& x, Arena& arena, hipStream_t s, int out_epilogue) const {
+        Pending p;
+        first_products(h, step, arena, s, p, false);
+        rest(p, step, x, arena, s, out_epilogue);
+    }
+    bool begin(NormedInput& h, const StepView& step, Arena& arena, hipStream_t s, Pending& pending) const override {
+        // (few rows in bfloat16: each of the two products norms its input itself, and no norm kernel runs)
+        first_products(h, step, arena, s, pending, dtype_ == BF16 && step.n_tokens <= tuning().ln_fuse_max_rows);
+        return true;
+    }
+    void finish(const Pending& pending, const StepView& step, const Tensor2& x, Arena& arena, hipStream_t s) const override {
+        rest(pending, step, x, arena, s, ADD_RESIDUAL);
+    }
+    // pending.a: the router's logits (fp32), pending.b: the experts' joined first product
+    void first_products(NormedInput& h, const StepView& step, Arena& arena, hipStream_t s, Pending& p, bool norm_inside) const {
         const int T = step.n_tokens, N = up_.out_features(), R = router_.out_features();
-        const Tensor2& in = h.tensor(arena, s);
         const int lde = (R + 3) / 4 * 4;
-        Tensor2 logits(arena.take(static_cast<size_t>(T) * lde * 4), F32, T, R, lde);
-        router_(in, logits, STORE_F32, nullptr, s);
-        StageTimes::get().mark("router", s);
-        Tensor2 inner = arena.tensor(dtype_, T, N);
-        up_(in, inner, STORE, nullptr, s);
+        p.a = Tensor2(arena.take(static_cast<size_t>(T) * lde * 4), F32, T, R, lde);
+        p.b = arena.tensor(dtype_, T, N);
+        if (norm_inside) {
+            h.linear(router_, p.a, STORE_F32, nullptr, arena, s);
+            StageTimes::get().mark("router", s);
+            h.linear(up_, p.b, STORE, nullptr, arena, s);
+        } else {
+            const Tensor2& in = h.tensor(arena, s);
+            router_(in, p.a, STORE_F32, nullptr, s);
+            StageTimes::get().mark("router", s);
+            up_(in, p.b, STORE, nullptr, s);
+        }
         StageTimes::get().mark("fc1", s);
+    }
+    void rest(const Pending& p, const StepView& step, const Tensor2& x, Arena& arena, hipStream_t s, int out_epilogue) const {
         if (gated_) {
-            Tensor2 act = arena.tensor(dtype_, T, down_.in_features());
-            moe_glu_act(inner, logits, glu_, act, s);
+            Tensor2 act = arena.tensor(dtype_, step.n_tokens, down_.in_features());
+            moe_glu_act(p.b, p.a, glu_, act, s);
             down_(act, x, out_epilogue, nullptr, s);
         } else {
-            moe_act(inner, logits, ff_, top_, scale_, inner, nullptr, s);            // in place
-            down_(inner, x, out_epilogue, nullptr, s);
+            moe_act(p.b, p.a, ff_, top_, scale_, p.b, nullptr, s);            // in place
+            down_(p.b, x, out_epilogue, nullptr, s);
         }
         StageTimes::get().mark("fc2", s);
     }

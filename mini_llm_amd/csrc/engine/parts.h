@@ -279,6 +279,19 @@ public:
         fill_zero(x, s);
         forward(h, step, x, arena, s);
     }
+    // The same in two halves, for an arrangement whose sub-layers read ONE stream: begin() does everything that reads
+    // the input (the first products, with the norm inside them where the kernels allow) and leaves what it made in the
+    // arena, in `pending`; finish() does the rest and adds into x, after somebody else may have changed x. What
+    // begin() took from the arena must still be there when finish() runs. False from begin(): this kind has no halves,
+    // and nothing was done.
+    struct Pending { Tensor2 a, b; };
+    virtual bool begin(NormedInput& h, const StepView& step, Arena& arena, hipStream_t s, Pending& pending) const {
+        (void)h; (void)step; (void)arena; (void)s; (void)pending;
+        return false;
+    }
+    virtual void finish(const Pending& pending, const StepView& step, const Tensor2& x, Arena& arena, hipStream_t s) const {
+        (void)pending; (void)step; (void)x; (void)arena; (void)s;
+    }
     virtual size_t workspace_bytes(int tokens) const = 0;
     virtual void reserve(int max_seqs, hipStream_t s) const { (void)max_seqs; (void)s; }
     virtual void add_cost(StepCost&) const {}

@@ -275,8 +275,9 @@ private:
 
 // Mixer and feed-forward side by side, each behind a norm of its own, both reading the SAME stream:
 //   x += mixer(norm1(x)) + ff(norm2(x))
-// The feed-forward's input is normed before the mixer adds its result into the stream; then both add theirs. Norms:
-// [norm1] or [norm1, norm2].
+// The feed-forward's input is normed before the mixer adds its result into the stream; then both add theirs. For few
+// rows a feed-forward that has halves (FeedForward::begin / finish) runs its first products, with the norm inside
+// them, before the mixer and the rest behind it, and no norm kernel runs. Norms: [norm1] or [norm1, norm2].
 class ParallelNormBlock final : public Block {
 public:
     ParallelNormBlock(std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f, std::vector<std::unique_ptr<Norm>> norms, const Params&)
@@ -290,23 +291,34 @@ public:
     void forward(const Tensor2& x, const StepView& step, const CacheView& cache, bool write, Arena& arena,
                  hipStream_t s) const override {
         const size_t outer = arena.mark();
+        // Few rows: the feed-forward's first products run before the mixer, with the norm inside them, and the rest
+        // behind it; otherwise its input is normed before the mixer changes x.
         Tensor2 h2;
-        if (ff_) h2 = norm2_->forward(x, nullptr, static_cast<int>(x.rows), arena, s);      // (before the mixer changes x)
+        FeedForward::Pending pending;
+        bool halves = false;
+        if (ff_ && x.rows <= tuning().ln_fuse_max_rows) {
+            NormedInput h(*norm2_, x);
+            halves = ff_->begin(h, step, arena, s, pending);
+        }
+        if (ff_ && !halves) h2 = norm2_->forward(x, nullptr, static_cast<int>(x.rows), arena, s);
         const size_t mark = arena.mark();
         {
             NormedInput h(*norm1_, x);
             mixer_->forward(h, step, cache, x, write, arena, s);
         }
         arena.release(mark);
-        if (ff_) {
+        if (halves) {
+            ff_->finish(pending, step, x, arena, s);
+        } else if (ff_) {
             NormedInput h(h2);
             ff_->forward(h, step, x, arena, s);
         }
         arena.release(outer);
     }
     size_t workspace_bytes(int tokens) const override {
+        // (what the feed-forward's first half leaves in the arena stays there while the mixer runs)
         size_t a = mixer_->workspace_bytes(tokens) + 2 * norm1_->workspace_bytes(tokens);
-        if (ff_) a = std::max(a, ff_->workspace_bytes(tokens)) + 2 * norm2_->workspace_bytes(tokens);
+        if (ff_) a += ff_->workspace_bytes(tokens) + 2 * norm2_->workspace_bytes(tokens);
         return a + 1024;
     }
     CacheNeed cache_need() const override { return mixer_->cache_need(); }

@@ -197,11 +197,19 @@ public:
         if (gate_up_.out_features() != 2 * down_.in_features()) fail("gated_mlp: the products' shapes do not fit");
     }
     void forward(NormedInput& h, const StepView& step, const Tensor2& x, Arena& arena, hipStream_t s) const override {
-        const int T = step.n_tokens, F = down_.in_features();
-        Tensor2 gu = arena.tensor(dtype_, T, 2 * F), a = arena.tensor(dtype_, T, F);
-        h.linear(gate_up_, gu, STORE, nullptr, arena, s);
+        Pending p;
+        begin(h, step, arena, s, p);
+        finish(p, step, x, arena, s);
+    }
+    bool begin(NormedInput& h, const StepView& step, Arena& arena, hipStream_t s, Pending& pending) const override {
+        pending.a = arena.tensor(dtype_, step.n_tokens, 2 * down_.in_features());
+        h.linear(gate_up_, pending.a, STORE, nullptr, arena, s);
         StageTimes::get().mark("fc1", s);
-        glu_act(gu, act_, a, s);
+        return true;
+    }
+    void finish(const Pending& pending, const StepView& step, const Tensor2& x, Arena& arena, hipStream_t s) const override {
+        Tensor2 a = arena.tensor(dtype_, step.n_tokens, down_.in_features());
+        glu_act(pending.a, act_, a, s);
         down_(a, x, ADD_RESIDUAL, nullptr, s);
         StageTimes::get().mark("fc2", s);
     }

@@ -116,7 +116,7 @@ struct SunulornConfig {
                 if (x.vdim != x.dim) throw ConfigError("config.json: " + where + "the values are the keys: vdim must equal dim");
                 if (const Json* taps = m.find("conv")) {
                     if (!taps->is_null()) {
-                        x.taps = need_int(m, "conv", where);
+                        x.taps = need_int(m, "conv", where, 0);           // (0: none, as when the key is absent)
                         if (x.taps > 16) throw ConfigError("config.json: " + where + "a convolution of more than 16 taps is not supported");
                     }
                 }

@@ -46,10 +46,11 @@ def test_keys_that_may_be_absent_have_the_plain_meaning():
     m.pop("kv_heads"); m.pop("vdim"); m.pop("mask"); m.pop("rot")
     cfg["layers"][1]["mlp"].pop("kind")          # dense
     cfg["layers"][1]["mixer"].pop("conv")
+    cfg["layers"][4]["mixer"]["conv"] = 0            # (no taps: no convolution either)
     cfg.pop("embedding")
     shapes = {t["name"]: t["shape"] for t in describe_config(cfg)["tensors"]}
     assert shapes["l2.mix.k"] == [heads * dim, 64] and shapes["l2.mix.v"] == [heads * dim, 64]
-    assert "l1.mlp.gate" in shapes and "l1.mix.q.conv" not in shapes
+    assert "l1.mlp.gate" in shapes and "l1.mix.q.conv" not in shapes and "l4.mix.k.conv" not in shapes
 
 
 @pytest.mark.parametrize("change, message", [

@@ -61,14 +61,14 @@ def test_each_mechanism_alone(dirs, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["MIXED_A", "MIXED_B", "ODD"])
+@pytest.mark.parametrize("name", ["MIXED_A", "MIXED_B", "ODD", "UNUSUAL"])
 @pytest.mark.parametrize("family", ["whole", "decode", "chunks", "mixed"])
 def test_schedule_families_match_plain(dirs, name, family, dtype):
     """Each request whole; most of it at once and the rest token by token; portions down to two tokens; up to
     four live requests in mixed batches. The pool holds just the peak of live tokens and there are four state
     slots for eight requests, so pages and slots are used again (and were filled with NaN before)."""
     cfg, d = getattr(sc, name), dirs(name)
-    reqs = sc.requests(cfg["vocab"], [1, 2, 3, 4, 5, 29, 64, 71] + ([150] if name == "ODD" else []), seed=11)
+    reqs = sc.requests(cfg["vocab"], [1, 2, 3, 4, 5, 29, 64, 71] + ([150] if name in ("ODD", "UNUSUAL") else []), seed=11)
     steps = _families(reqs, seed=2)[family]
     n_pages = ru.peak_tokens(steps) // 4
     runner = _runner(d, dtype, n_pages)
