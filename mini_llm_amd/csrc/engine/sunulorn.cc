@@ -263,12 +263,21 @@ void sunulorn_assemble(const Json& config, const std::map<std::string, Tensor2>&
         // Value heads narrower than the keys are made as wide: zero rows in the values' projection (and the gate's), zero
         // columns in the output projection. The result is the same, and the attention kernels that every model shares
         // (key tiles on the matrix cores, split keys) take keys and values of one width only.
+        // Value heads WIDER than the keys: the queries' and keys' heads get zero columns instead (zero rows in their
+        // projections and biases); the dot products are the same. Where queries and keys are scaled to unit root mean
+        // square over the head, the wider head's mean is dim / d times the true one, so eps * dim / d stands for eps
+        // and the normed vectors come out sqrt(d / dim) times too long, which scale * dim / d takes back:
+        //   x / sqrt(sum / d + eps dim / d) = sqrt(d / dim) x / sqrt(sum / dim + eps).
         const int64_t e = (x.vdim < x.dim && x.dim % 16 == 0) ? x.dim : x.vdim;
+        const int64_t d = (x.vdim > x.dim && x.vdim % 16 == 0 && x.kind != MixerConfig::ConvAttention) ? x.vdim : x.dim;
         auto widened_rows = [&](const Tensor2& w) { return e == x.vdim ? w : out.store.pad_row_blocks(w, x.vdim, e); };
+        auto widened_keys = [&](const Tensor2& w) { return d == x.dim ? w : out.store.pad_row_blocks(w, x.dim, d); };
+        const double shrink = static_cast<double>(x.dim) / static_cast<double>(d);
+        const bool unit_norm = x.kind == MixerConfig::WindowAttention;
         Params p;
         p.num["heads"] = static_cast<double>(x.heads); p.num["kv_heads"] = static_cast<double>(x.kv_heads);
-        p.num["dim"] = static_cast<double>(x.dim); p.num["value_dim"] = static_cast<double>(e);
-        p.num["scale"] = x.scale; p.num["eps"] = c.eps; p.num["dtype"] = dtype;
+        p.num["dim"] = static_cast<double>(d); p.num["value_dim"] = static_cast<double>(e);
+        p.num["scale"] = unit_norm ? x.scale * shrink : x.scale; p.num["eps"] = unit_norm ? c.eps * shrink : c.eps; p.num["dtype"] = dtype;
         p.str["qk_norm"] = "none";
         p.tensor["out.weight"] = e == x.vdim ? t.at(M + "o") : out.store.pad_col_blocks(t.at(M + "o"), x.vdim, e);
         if (x.kind == MixerConfig::ConvAttention) {
@@ -283,9 +292,9 @@ void sunulorn_assemble(const Json& config, const std::map<std::string, Tensor2>&
             p.str["qk_norm"] = "unit_after";
             p.num["window"] = static_cast<double>(x.window); p.num["keep_first"] = static_cast<double>(x.window > 0 ? x.keep_first : 0);
             p.num["gated"] = 1;
-            p.tensor["in.weight"] = out.store.join_rows({t.at(M + "q"), t.at(M + "k"), widened_rows(t.at(M + "v")), widened_rows(t.at(M + "g"))});
+            p.tensor["in.weight"] = out.store.join_rows({widened_keys(t.at(M + "q")), widened_keys(t.at(M + "k")), widened_rows(t.at(M + "v")), widened_rows(t.at(M + "g"))});
             // (the gate's projection has no bias)
-            p.tensor["in.bias"] = out.store.join_rows({column(t.at(M + "q.b")), column(t.at(M + "k.b")), widened_rows(column(t.at(M + "v.b"))), column(out.store.zeros(x.heads * e))});
+            p.tensor["in.bias"] = out.store.join_rows({widened_keys(column(t.at(M + "q.b"))), widened_keys(column(t.at(M + "k.b"))), widened_rows(column(t.at(M + "v.b"))), column(out.store.zeros(x.heads * e))});
             p.tensor["out.bias"] = t.at(M + "o.b");
         } else {
             p.num["gated"] = 1; p.num["gate_per_head"] = 1;
@@ -295,11 +304,11 @@ void sunulorn_assemble(const Json& config, const std::map<std::string, Tensor2>&
             p.tensor["distance_slope"] = out.store.upload(slopes, 1, static_cast<int64_t>(slopes.size()), F32);
             if (x.kv_from >= 0) {
                 p.num["shared_kv"] = 1;
-                p.tensor["in.weight"] = out.store.join_rows({t.at(M + "q"), t.at(M + "g")});
-                p.tensor["in.bias"] = out.store.join_rows({column(t.at(M + "q.b")), column(out.store.zeros(x.heads))});
+                p.tensor["in.weight"] = out.store.join_rows({widened_keys(t.at(M + "q")), t.at(M + "g")});
+                p.tensor["in.bias"] = out.store.join_rows({widened_keys(column(t.at(M + "q.b"))), column(out.store.zeros(x.heads))});
             } else {
-                p.tensor["in.weight"] = out.store.join_rows({t.at(M + "q"), t.at(M + "k"), widened_rows(t.at(M + "v")), t.at(M + "g")});
-                p.tensor["in.bias"] = out.store.join_rows({column(t.at(M + "q.b")), column(t.at(M + "k.b")), widened_rows(column(t.at(M + "v.b"))), column(out.store.zeros(x.heads))});
+                p.tensor["in.weight"] = out.store.join_rows({widened_keys(t.at(M + "q")), widened_keys(t.at(M + "k")), widened_rows(t.at(M + "v")), t.at(M + "g")});
+                p.tensor["in.bias"] = out.store.join_rows({widened_keys(column(t.at(M + "q.b"))), widened_keys(column(t.at(M + "k.b"))), widened_rows(column(t.at(M + "v.b"))), column(out.store.zeros(x.heads))});
             }
         }
         std::unique_ptr<Mixer> mixer = build_mixer("scored_attention", p);

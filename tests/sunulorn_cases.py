@@ -114,14 +114,15 @@ ODD = model([
     sink_attention(heads=2, kv_heads=1, dim=7, vdim=5, mlp=dense(19)),
     sink_attention(heads=2, kv_heads=1, dim=7, vdim=5, kv_from=2, mlp=moe(experts=3, top=1, ff=9, shared=None)),
 ], vocab=101, width=43)
-# head sizes between the kernels' own: keys of 96 with narrower values (widened, 32-bit tiles), keys of 80 with WIDER
-# values (the row kernel), keys and values of 48 read by a second layer, six heads over three
+# head sizes between the kernels' own: keys of 96 with narrower values (the values widened), keys of 80 and of 48 with
+# WIDER values (the keys widened, with the unit norm's eps and the score's scale adjusted), the latter read by a second
+# layer, six heads over three
 UNUSUAL = model([
     window_attention(heads=2, kv_heads=1, dim=96, vdim=32, window=40, keep=9, dims=48, mlp=dense(80)),
     window_attention(heads=2, kv_heads=2, dim=80, vdim=112, window=21, keep=33, dims=80, mlp=moe(experts=9, top=3, ff=40, shared=24)),
-    sink_attention(heads=6, kv_heads=3, dim=48, vdim=48, mlp=dense(64)),
+    sink_attention(heads=6, kv_heads=3, dim=48, vdim=64, mlp=dense(64)),
     conv_attention(heads=2, kv_heads=1, dim=96, taps=2, dims=64, mlp=moe(experts=2, top=1, ff=56, shared=None)),
-    sink_attention(heads=6, kv_heads=3, dim=48, vdim=48, kv_from=2, mlp=dense(64)),
+    sink_attention(heads=6, kv_heads=3, dim=48, vdim=64, kv_from=2, mlp=dense(64)),
 ], vocab=333, width=96)
 # the sizes of a larger model's layers: heads of 64 and 128, pages of many sizes
 LARGER = model([
