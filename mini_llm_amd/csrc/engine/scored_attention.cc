@@ -64,7 +64,6 @@ public:
         if (H < 1 || G < 1 || H % G != 0 || d < 1 || dv < 1) fail("scored_attention: %d heads over %d key/value heads of %d / %d do not fit", H, G, d, dv);
         if (sh_.window < 0 || sh_.chunk < 0 || (sh_.window > 0 && sh_.chunk > 0)) fail("scored_attention: a window or a chunk, not both");
         if (sh_.keep_first < 0 || (sh_.keep_first > 0 && sh_.window <= 0)) fail("scored_attention: kept first positions go with a sliding window");
-
         if (values_from_keys_ && dv != d) fail("scored_attention: values taken from the keys have the keys' width, %d, not %d", d, dv);
         if (sh_.rot_dims < 0 || sh_.rot_dims % 2 != 0 || sh_.rot_dims > d) fail("scored_attention: %d turned columns of %d: even and at most the head", sh_.rot_dims, d);
         const std::string& mode = p.string("qk_norm");

@@ -99,7 +99,7 @@ SINK_SOFT = model([conv_attention(scale=0.02), sink_attention(scale=0.02)], widt
 # the same at the head sizes that the matrix-core tiles and the split-key kernel take in bfloat16 (32, 64, 128; keys and
 # values of one width), one layer each so that a row shows its own mask
 PEAKED_TILES_32 = model([window_attention(window=9, keep=3, scale=0.8, heads=4, kv_heads=2, dim=32, vdim=32, dims=32)], width=64)
-PEAKED_TILES_64 = model([window_attention(window=70, keep=20, scale=0.6, heads=2, kv_heads=1, dim=64, vdim=64, dims=32)], width=64)
+PEAKED_TILES_64 = model([window_attention(window=70, keep=23, scale=0.6, heads=2, kv_heads=1, dim=64, vdim=64, dims=32)], width=64)
 PEAKED_TILES_128 = model([window_attention(window=3, keep=130, scale=0.4, heads=2, kv_heads=2, dim=128, vdim=128, dims=64)], width=32)
 SINK_TILES_64 = model([sink_attention(heads=4, kv_heads=2, dim=64, vdim=64, scale=0.5)], width=64)
 CONV_TILES_128 = model([conv_attention(heads=2, kv_heads=1, dim=128, taps=4, dims=32, scale=0.3)], width=64)
@@ -127,7 +127,7 @@ UNUSUAL = model([
 # the sizes of a larger model's layers: heads of 64 and 128, pages of many sizes
 LARGER = model([
     conv_attention(heads=4, kv_heads=2, dim=64, taps=4, dims=32, mlp=moe(experts=6, top=2, ff=96, shared=160)),
-    window_attention(heads=4, kv_heads=2, dim=64, vdim=64, window=100, keep=20, dims=64, mlp=dense(384)),
+    window_attention(heads=4, kv_heads=2, dim=64, vdim=64, window=100, keep=26, dims=64, mlp=dense(384)),
     sink_attention(heads=2, kv_heads=1, dim=128, vdim=128, mlp=moe(experts=6, top=2, ff=96, shared=160)),
     sink_attention(heads=2, kv_heads=1, dim=128, vdim=128, kv_from=2),
     window_attention(heads=8, kv_heads=2, dim=32, vdim=48, window=150, keep=17, dims=16, mlp=dense(256)),
