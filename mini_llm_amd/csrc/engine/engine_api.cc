@@ -60,7 +60,7 @@ unsigned long long mllm_scratch_bytes(void) {
 }
 int mllm_release_scratch(hipStream_t stream) { return guarded([&] { release_scratch(stream); }); }
 // name: "decode_shape" (nsplit, waves; 0, 0 = automatic), "unmerged_shape", "merge_max_rows" (a), "ln_fuse_max_rows" (a), "long_context_splits" (a: 0 off, 1 on),
-// "latent_tiles", "scored_shared_kernels" (a: 0 off, 1 on)
+// "latent_tiles", "scored_shared_kernels" (a: 0 off, 1 on), "halves_max_width" (a)
 int mllm_set_tuning(const char* name, int a, int b) {
     return guarded([&] {
         Tuning& t = tuning();
@@ -72,6 +72,7 @@ int mllm_set_tuning(const char* name, int a, int b) {
         else if (n == "long_context_splits") t.long_context_splits = a;
         else if (n == "latent_tiles") t.latent_tiles = a;
         else if (n == "scored_shared_kernels") t.scored_shared_kernels = a;
+        else if (n == "halves_max_width") t.halves_max_width = a;
         else if (n == "reset_seen") t.seen = Tuning::Seen();
         else fail("unknown tuning value '%s'", name);
     });

@@ -117,6 +117,10 @@ struct Tuning {
     int ln_fuse_max_rows = 32;                        // rows up to which the norm is fused into the few-row product
     int latent_tiles = 1;                             // 1: latent attention's prompt portions may run on the matrix cores
     int scored_shared_kernels = 1;                    // 1: attention with shaped scores may run on the kernels the plain attention runs on
+    int halves_max_width = 1024;                      // stream widths up to which a block whose sub-layers read one stream runs the
+                                                      // feed-forward's first products, with the norm inside, in front of the mixer
+                                                      // (wider: every workgroup of a wide product redoing the norm costs more than the
+                                                      // norm's own kernel; at width 1,600 the halves lost 5 % of a decode step)
     // what the ops chose since the last reset (tests read it back instead of trusting the thresholds)
     struct Seen {
         int max_decode_splits = 0;                    // most workgroups a (token, head) pair's keys were split over

@@ -296,7 +296,7 @@ public:
         Tensor2 h2;
         FeedForward::Pending pending;
         bool halves = false;
-        if (ff_ && x.rows <= tuning().ln_fuse_max_rows) {
+        if (ff_ && x.rows <= tuning().ln_fuse_max_rows && x.cols <= tuning().halves_max_width) {
             NormedInput h(*norm2_, x);
             halves = ff_->begin(h, step, arena, s, pending);
         }
